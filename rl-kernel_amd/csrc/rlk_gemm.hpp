@@ -1,0 +1,278 @@
+// MFMA tile GEMM mainloop for gfx950 (CDNA4), shared by the four contraction kernels of the
+// fused linear-logprob path (forward logits tile, dZ recompute, dH, dW).
+//
+// One workgroup = 256 threads = 4 wavefronts arranged 2 (M) x 2 (N).  The workgroup computes a
+// (2*TM*32) x (2*TN*32) tile D = A * B^T-like contraction over K with v_mfma_f32_32x32x16
+// (bf16 or f16 inputs, fp32 accumulate); each wavefront owns TM x TN MFMA tiles of 32x32.
+//
+// Operands are described by (base pointer at the tile origin, leading dimension, valid rows):
+//   * "K-contiguous" operand: memory is [row][k] with k fastest (W and hidden in the forward).
+//   * "K-major" operand:      memory is [k][row] with row fastest (W in dH, dZ and hidden in dW).
+//     Its fragments are fetched from LDS with the gfx950 transposing read
+//     ds_read_b64_tr_b16, so no transposed copy of any tensor is ever written to HBM.
+//
+// Pipeline: global -> registers -> LDS (double buffered, one barrier per K step) -> MFMA.
+// Loads never leave the valid part of the tensor: row indices are clamped, and K chunks beyond
+// the valid K range are replaced by zeros, so no out-of-bounds address is ever formed.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rlk {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+
+#define RLK_LDS __attribute__((address_space(3)))
+
+constexpr int kThreads = 256;
+
+struct Bf16 {
+    static constexpr int kId = 0;
+    using scalar = __bf16;
+    __device__ static inline f32x16_t mfma(u32x4_t a, u32x4_t b, f32x16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    __device__ static inline uint16_t from_float(float x)
+    {
+        return __builtin_bit_cast(uint16_t, static_cast<__bf16>(x));
+    }
+    __device__ static inline float to_float(uint16_t x)
+    {
+        return __builtin_bit_cast(float, static_cast<uint32_t>(x) << 16);
+    }
+};
+
+struct F16 {
+    static constexpr int kId = 1;
+    using scalar = _Float16;
+    __device__ static inline f32x16_t mfma(u32x4_t a, u32x4_t b, f32x16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                      __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    __device__ static inline uint16_t from_float(float x)
+    {
+        return __builtin_bit_cast(uint16_t, static_cast<_Float16>(x));
+    }
+    __device__ static inline float to_float(uint16_t x)
+    {
+        return static_cast<float>(__builtin_bit_cast(_Float16, x));
+    }
+};
+
+// 16-bit matrix operand of one workgroup tile.
+struct Operand {
+    const uint16_t* base;  // element (row 0, k 0) of the tile
+    int64_t ld;            // elements between consecutive memory lines
+    int rows;              // valid tile rows from the origin (>= 1)
+};
+
+// LDS geometry of one operand tile.
+template <bool KMAJOR, int ROWS, int BK>
+struct TileGeom {
+    // K-contiguous: one line per tile row, BK elements + 16 B pad (conflict-free b128 fragment reads).
+    // K-major:      one line per k, ROWS elements + 64 B pad (conflict-free transposing reads).
+    static constexpr int kPitch = KMAJOR ? (ROWS * 2 + 64) : (BK * 2 + 16);
+    static constexpr int kLines = KMAJOR ? BK : ROWS;
+    static constexpr int kBytes = kPitch * kLines;
+    static constexpr int kChunksPerLine = KMAJOR ? (ROWS / 8) : (BK / 8);
+    static constexpr int kLinesPerPass = kThreads / kChunksPerLine;
+    static constexpr int kPasses = kLines / kLinesPerPass;
+    static_assert(kLines % kLinesPerPass == 0, "tile does not divide over 256 threads");
+};
+
+template <bool KMAJOR, int ROWS, int BK>
+struct TileIO {
+    using G = TileGeom<KMAJOR, ROWS, BK>;
+
+    // Per-thread addressing of one operand: a uniform base pointer plus 32-bit byte offsets of
+    // this thread's chunks at K step 0 (already clamped into the valid part of the tensor).
+    const char* base;
+    uint32_t off[G::kPasses];
+    uint32_t step;  // byte advance per K step
+
+    __device__ inline void init(const Operand& op, int K)
+    {
+        const int t = threadIdx.x;
+        const int chunk = t % G::kChunksPerLine;
+        const int line0 = t / G::kChunksPerLine;
+        base = reinterpret_cast<const char*>(op.base);
+        const uint32_t ld = static_cast<uint32_t>(op.ld);
+        step = KMAJOR ? static_cast<uint32_t>(BK) * ld * 2u : static_cast<uint32_t>(BK) * 2u;
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int line = p * G::kLinesPerPass + line0;
+            if (KMAJOR) {
+                const int k = line < K ? line : K - 1;
+                const int r = chunk * 8 < op.rows ? chunk * 8 : 0;
+                off[p] = (static_cast<uint32_t>(k) * ld + static_cast<uint32_t>(r)) * 2u;
+            } else {
+                const int r = line < op.rows ? line : op.rows - 1;
+                const int k = chunk * 8 < K ? chunk * 8 : 0;
+                off[p] = (static_cast<uint32_t>(r) * ld + static_cast<uint32_t>(k)) * 2u;
+            }
+        }
+    }
+
+    // Fetch this thread's 16-byte chunks of K step kt.  CHECKED: chunks at k >= K come back as
+    // zeros (only needed for the last, partial K step).
+    template <bool CHECKED>
+    __device__ inline void load(int kt, int K, u32x4_t (&reg)[G::kPasses]) const
+    {
+        const int t = threadIdx.x;
+        const int chunk = t % G::kChunksPerLine;
+        const int line0 = t / G::kChunksPerLine;
+        const uint32_t adv = static_cast<uint32_t>(kt) * step;
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            if (CHECKED) {
+                const int k = kt * BK + (KMAJOR ? p * G::kLinesPerPass + line0 : chunk * 8);
+                const bool live = k < K;
+                const uint32_t o = live ? off[p] + adv : off[p];
+                u32x4_t v = *reinterpret_cast<const u32x4_t*>(base + o);
+                if (!live) v = u32x4_t{0u, 0u, 0u, 0u};
+                reg[p] = v;
+            } else {
+                reg[p] = *reinterpret_cast<const u32x4_t*>(base + (off[p] + adv));
+            }
+        }
+    }
+
+    __device__ static inline void store(char* lds, const u32x4_t (&reg)[G::kPasses])
+    {
+        const int t = threadIdx.x;
+        const int chunk = t % G::kChunksPerLine;
+        const int line0 = t / G::kChunksPerLine;
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int line = p * G::kLinesPerPass + line0;
+            *reinterpret_cast<u32x4_t*>(lds + line * G::kPitch + chunk * 16) = reg[p];
+        }
+    }
+
+    // MFMA 32x32x16 operand fragment: lane l holds row (row0 + l%32), k = kk*16 + 8*(l/32) + 0..7.
+    __device__ static inline u32x4_t frag(const char* lds, int row0, int kk)
+    {
+        const int l = threadIdx.x & 63;
+        if (KMAJOR) {
+            // ds_read_b64_tr_b16: inside each group of 16 lanes, lane 4a+b supplies the address of
+            // 4 consecutive rows (4b..4b+3) of k-line a; lane i receives row i of k-lines 0..3.
+            const int a = (l & 15) >> 2;
+            const int b = l & 3;
+            const int kline = kk * 16 + 8 * (l >> 5) + a;
+            const int col = row0 + 16 * ((l >> 4) & 1) + 4 * b;
+            const char* p0 = lds + kline * G::kPitch + col * 2;
+            const char* p1 = p0 + 4 * G::kPitch;
+            s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RLK_LDS s16x4_t*)(p0));
+            s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RLK_LDS s16x4_t*)(p1));
+            u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
+            u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
+            return u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y};
+        } else {
+            const char* p = lds + (row0 + (l & 31)) * G::kPitch + (kk * 16 + 8 * (l >> 5)) * 2;
+            return *reinterpret_cast<const u32x4_t*>(p);
+        }
+    }
+};
+
+// Workgroup tile contraction.  acc[i][j] (+)= A rows x B rows over k in [0, K).
+// smem must hold 2 * (A tile + B tile) bytes.  All 256 threads must call it (it barriers).
+template <class T, bool A_KMAJOR, bool B_KMAJOR, int TM, int TN, int BK>
+struct TileGemm {
+    static constexpr int BM = 2 * TM * 32;
+    static constexpr int BN = 2 * TN * 32;
+    using IOA = TileIO<A_KMAJOR, BM, BK>;
+    using IOB = TileIO<B_KMAJOR, BN, BK>;
+    static constexpr int kStageBytes = IOA::G::kBytes + IOB::G::kBytes;
+    static constexpr int kSmemBytes = 2 * kStageBytes;
+
+    __device__ static inline void run(const Operand& A, const Operand& B, int K,
+                                      f32x16_t (&acc)[TM][TN], char* smem)
+    {
+        const int wave = threadIdx.x >> 6;
+        const int wm = wave >> 1;
+        const int wn = wave & 1;
+        u32x4_t ra[IOA::G::kPasses];
+        u32x4_t rb[IOB::G::kPasses];
+
+        IOA la;
+        IOB lb;
+        la.init(A, K);
+        lb.init(B, K);
+        const int nk = (K + BK - 1) / BK;
+        const int nfull = K / BK;  // K steps that need no bounds check
+        la.template load<true>(0, K, ra);
+        lb.template load<true>(0, K, rb);
+        IOA::store(smem, ra);
+        IOB::store(smem + IOA::G::kBytes, rb);
+        __syncthreads();
+
+        for (int kt = 0; kt < nk; ++kt) {
+            char* cur = smem + (kt & 1) * kStageBytes;
+            char* nxt = smem + ((kt + 1) & 1) * kStageBytes;
+            const bool more = kt + 1 < nk;
+            if (more) {
+                if (kt + 1 < nfull) {
+                    la.template load<false>(kt + 1, K, ra);
+                    lb.template load<false>(kt + 1, K, rb);
+                } else {
+                    la.template load<true>(kt + 1, K, ra);
+                    lb.template load<true>(kt + 1, K, rb);
+                }
+            }
+            const char* sa = cur;
+            const char* sb = cur + IOA::G::kBytes;
+#pragma unroll
+            for (int kk = 0; kk < BK / 16; ++kk) {
+                u32x4_t fa[TM];
+                u32x4_t fb[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[i] = IOA::frag(sa, wm * (TM * 32) + i * 32, kk);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) fb[j] = IOB::frag(sb, wn * (TN * 32) + j * 32, kk);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j] = T::mfma(fa[i], fb[j], acc[i][j]);
+            }
+            if (more) {
+                IOA::store(nxt, ra);
+                IOB::store(nxt + IOA::G::kBytes, rb);
+            }
+            __syncthreads();
+        }
+    }
+};
+
+// Row of the 32x32 accumulator held in register r of lane l: D[8*(r/4) + 4*(l/32) + r%4][l%32].
+__device__ inline int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+// Map a linear workgroup id to a tile so that the 32 workgroups resident on one XCD (ids equal
+// modulo 8 run on the same XCD and share its L2) cover a compact patch of `group` tile rows.
+__device__ inline void xcd_tile(int lin, int total, int gm, int gn, int group, int& tm, int& tn)
+{
+    const int per = total >> 3;
+    const int rem = total & 7;
+    const int xcd = lin & 7;
+    const int idx = lin >> 3;
+    const int seq = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    const int gsz = group * gn;
+    const int gid = seq / gsz;
+    const int first = gid * group;
+    const int rows = (gm - first) < group ? (gm - first) : group;
+    const int in = seq - gid * gsz;
+    tm = first + in % rows;
+    tn = in / rows;
+}
+
+}  // namespace rlk

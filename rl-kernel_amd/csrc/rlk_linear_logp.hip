@@ -1,0 +1,909 @@
+// Fused linear -> selected-token log-prob for gfx950: forward (online logsumexp over vocab
+// tiles, logits never stored), split combine, and the recompute-based backward (dZ block,
+// dH and dW contractions).  All reductions run in a fixed order: same input, same bits.
+//
+// Orientation used by every kernel here: the MFMA "M" index lives in accumulator registers
+// (4 consecutive rows per register quad), the "N" index is the lane (column l % 32).  In the
+// forward and in the dZ recompute M = vocab and N = token, so one lane owns whole token columns
+// and the softmax reduction over vocab is a plain in-register loop with no cross-lane traffic.
+#include "rlk_common.hpp"
+#include "rlk_gemm.hpp"
+
+namespace rlk {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// ------------------------------------------------------------------------------------------- //
+// Forward
+// ------------------------------------------------------------------------------------------- //
+struct FwdArgs {
+    const uint16_t* hidden;   // [N][H]
+    const uint16_t* weight;   // [V][H]   (local vocab shard)
+    const float* bias;        // [V] or null
+    const int64_t* targets;   // [N] global ids
+    float* part_m;            // [n_split][N] running max (log2 domain)
+    float* part_s;            // [n_split][N] running sum of 2^(z - max)
+    float* part_z;            // [n_split][N] captured target logit (log2 domain), 0 if not owned
+    int N;
+    int H;
+    int V;
+    int64_t vocab_start;
+    int n_split;     // splits handled by this launch
+    int split_lo;    // first slot of the partial arrays this launch writes
+    int row_blocks;
+    int tile_lo;     // first vocab tile of this launch
+    int vtiles;      // vocab tiles of this launch
+    float scale2;    // log2(e) / temperature
+};
+
+// Online-softmax update of one wavefront slab (128 vocab rows x 128 tokens) held in `acc`.
+// GENERAL = false: no bias and no masked vocab rows (every tile full), the common case.
+// The target logit is picked up in the same pass that feeds the sum, so the captured value is
+// the very fp32 number that entered the softmax.
+template <bool GENERAL>
+__device__ inline void fwd_epilogue(const f32x16_t (&acc)[4][4], const FwdArgs& a, int vw, int lane,
+                                    const int (&tgt)[4], float (&m)[4], float (&s)[4],
+                                    float (&zt)[4])
+{
+    auto logit = [&](int i, int j, int r) -> float {
+        float z = acc[i][j][r];
+        if (GENERAL) {
+            const int v = vw + i * 32 + acc_row(r, lane);
+            if (a.bias != nullptr) z += a.bias[v < a.V ? v : a.V - 1];
+            if (v >= a.V) z = -INFINITY;
+        }
+        return z;
+    };
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, logit(i, j, r));
+        __builtin_amdgcn_sched_barrier(0);
+        tmax *= a.scale2;
+        const float mnew = fmaxf(m[j], tmax);
+        const float mref = mnew == -INFINITY ? 0.f : mnew;
+        // register index (i*16 + r) of the target row in this lane, or -1
+        const int tl = tgt[j] - vw;
+        const int x = tl & 31;
+        const int etgt = (static_cast<unsigned>(tl) < 128u && ((x >> 2) & 1) == (lane >> 5))
+                             ? ((tl >> 5) * 16 + (x >> 3) * 4 + (x & 3))
+                             : -1;
+        float sum = 0.f, zraw = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float z = logit(i, j, r);
+                sum += __builtin_amdgcn_exp2f(fmaf(z, a.scale2, -mref));
+                zraw = (etgt == i * 16 + r) ? z : zraw;
+            }
+        __builtin_amdgcn_sched_barrier(0);
+        s[j] = s[j] * __builtin_amdgcn_exp2f(m[j] - mref) + sum;
+        m[j] = mnew;
+        if (etgt >= 0) zt[j] = zraw * a.scale2;
+    }
+}
+
+// One workgroup = one block of 256 tokens x one contiguous range of vocab tiles.
+// GENERAL = false requires bias == null and covers only full vocab tiles [0, vtiles) split
+// n_split ways; GENERAL = true handles bias and/or masked rows over tiles [tile_lo, tile_lo+vtiles).
+template <class T, int BK, bool GENERAL>
+__global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
+{
+    constexpr int TM = 4, TN = 4;
+    using Gemm = TileGemm<T, false, false, TM, TN, BK>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    int tb, sp;
+    xcd_tile(blockIdx.x, a.row_blocks * a.n_split, a.row_blocks, a.n_split, 8, tb, sp);
+    // vocab tiles [t0, t1) of this split: the first (vtiles % n_split) splits take one extra.
+    const int base = a.vtiles / a.n_split, extra = a.vtiles % a.n_split;
+    const int t0 = a.tile_lo + sp * base + (sp < extra ? sp : extra);
+    const int t1 = t0 + base + (sp < extra ? 1 : 0);
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int tok0 = tb * 256;
+    const int tok_valid = min(256, a.N - tok0);
+
+    float m[TN], s[TN], zt[TN];
+    int tgt[TN];  // target id relative to the shard, -1 when not in [0, V)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        m[j] = -INFINITY;
+        s[j] = 0.f;
+        zt[j] = 0.f;
+        const int t = wn * 128 + j * 32 + (lane & 31);
+        int64_t g = a.targets[tok0 + (t < tok_valid ? t : tok_valid - 1)] - a.vocab_start;
+        tgt[j] = (g >= 0 && g < a.V) ? static_cast<int>(g) : -1;
+    }
+
+    Operand B{a.hidden + static_cast<int64_t>(tok0) * a.H, a.H, tok_valid};
+    for (int vt = t0; vt < t1; ++vt) {
+        const int v0 = vt * 256;
+        Operand A{a.weight + static_cast<int64_t>(v0) * a.H, a.H, min(256, a.V - v0)};
+        f32x16_t acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        Gemm::run(A, B, a.H, acc, smem);
+        fwd_epilogue<GENERAL>(acc, a, v0 + wm * 128, lane, tgt, m, s, zt);
+    }
+
+    // Merge the two half-wave row groups (same token, different vocab rows), then the two
+    // wavefronts along M through LDS, in a fixed order.
+    float* red = reinterpret_cast<float*>(smem);  // [2 (wm)][256 tokens][3]
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const float m2 = __shfl_xor(m[j], 32);
+        const float s2 = __shfl_xor(s[j], 32);
+        const float z2 = __shfl_xor(zt[j], 32);
+        const float mm = fmaxf(m[j], m2);
+        const float mref = mm == -INFINITY ? 0.f : mm;
+        const float lo_m = lane < 32 ? m[j] : m2, hi_m = lane < 32 ? m2 : m[j];
+        const float lo_s = lane < 32 ? s[j] : s2, hi_s = lane < 32 ? s2 : s[j];
+        const float ss = lo_s * __builtin_amdgcn_exp2f(lo_m - mref) +
+                         hi_s * __builtin_amdgcn_exp2f(hi_m - mref);
+        if (lane < 32) {
+            float* dst = red + ((wm * 256) + wn * 128 + j * 32 + lane) * 3;
+            dst[0] = mm;
+            dst[1] = ss;
+            dst[2] = zt[j] + z2;
+        }
+    }
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < tok_valid) {
+        const float* p0 = red + t * 3;
+        const float* p1 = red + (256 + t) * 3;
+        const float mm = fmaxf(p0[0], p1[0]);
+        const float mref = mm == -INFINITY ? 0.f : mm;
+        const float ss = p0[1] * __builtin_amdgcn_exp2f(p0[0] - mref) +
+                         p1[1] * __builtin_amdgcn_exp2f(p1[0] - mref);
+        const int64_t o = static_cast<int64_t>(a.split_lo + sp) * a.N + tok0 + t;
+        a.part_m[o] = mm;
+        a.part_s[o] = ss;
+        a.part_z[o] = p0[2] + p1[2];
+    }
+}
+
+struct CombineArgs {
+    const float* part_m;
+    const float* part_s;
+    const float* part_z;
+    const int64_t* targets;
+    float* logp;
+    float* lse;
+    int32_t* err_flag;
+    int N;
+    int V;
+    int n_split;
+    int64_t vocab_start;
+    int64_t ignore_index;
+    int use_ignore;
+    int strict;  // 1: a non-ignored target outside [vocab_start, vocab_start+V) raises err_flag
+};
+
+// M = max_s m_s ; S = sum_s s_s 2^(m_s - M) ; z_t = sum_s z_t,s ; lse = ln2 (M + log2 S).
+__global__ void linear_logp_combine_kernel(CombineArgs a)
+{
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= a.N) return;
+    float mm = -INFINITY;
+    for (int sp = 0; sp < a.n_split; ++sp) mm = fmaxf(mm, a.part_m[static_cast<int64_t>(sp) * a.N + n]);
+    float ss = 0.f, zz = 0.f;
+    for (int sp = 0; sp < a.n_split; ++sp) {
+        const int64_t o = static_cast<int64_t>(sp) * a.N + n;
+        ss += a.part_s[o] * exp2f(a.part_m[o] - mm);
+        zz += a.part_z[o];
+    }
+    const float lse2 = mm + log2f(ss);
+    const int64_t t = a.targets[n];
+    const bool ignored = a.use_ignore && t == a.ignore_index;
+    const int64_t tl = t - a.vocab_start;
+    const bool owned = tl >= 0 && tl < a.V;
+    if (!ignored && !owned && a.strict) *a.err_flag = 1;
+    a.lse[n] = lse2 * kLn2;
+    a.logp[n] = ignored ? 0.f : (zz - lse2) * kLn2;
+}
+
+// ------------------------------------------------------------------------------------------- //
+// Backward step 1: dZ block = g/T * (onehot - softmax) for a (token chunk) x (vocab piece)
+// ------------------------------------------------------------------------------------------- //
+struct DzArgs {
+    const uint16_t* hidden;  // chunk origin [tok][H]
+    const uint16_t* weight;  // piece origin [v][H]
+    const float* bias;       // piece origin or null
+    const int64_t* targets;  // chunk origin (global ids)
+    const float* lse;        // chunk origin (natural log)
+    const float* grad;       // chunk origin, upstream d/dlogp
+    const float* scales;     // [0] = loss_scale / temperature (device resident)
+    uint16_t* dz;            // [tok_tiles*256][ldz]
+    int64_t ldz;
+    int tok_valid;
+    int v_valid;
+    int H;
+    int tok_tiles;
+    int v_tiles;        // vocab tiles of this launch
+    int v_tile_lo;      // first vocab tile of this launch
+    int64_t v_global0;  // global id of the piece's first vocab row
+    int64_t ignore_index;
+    int use_ignore;
+    float scale2;
+};
+
+// GENERAL = false: no bias, every vocab tile of the launch is full.
+template <class T, int BK, bool GENERAL>
+__global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
+{
+    constexpr int TM = 4, TN = 4;
+    using Gemm = TileGemm<T, false, false, TM, TN, BK>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    int vt, tt;
+    xcd_tile(blockIdx.x, a.tok_tiles * a.v_tiles, a.v_tiles, a.tok_tiles, 8, vt, tt);
+    vt += a.v_tile_lo;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int tok0 = tt * 256, v0 = vt * 256;
+    const int tok_rows = min(256, a.tok_valid - tok0);
+    const int v_rows = min(256, a.v_valid - v0);
+
+    Operand A{a.weight + static_cast<int64_t>(v0) * a.H, a.H, v_rows};
+    Operand B{a.hidden + static_cast<int64_t>(tok0) * a.H, a.H, tok_rows};
+    f32x16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    Gemm::run(A, B, a.H, acc, smem);
+
+    const float gscale = a.scales[0];
+    const int vw = v0 + wm * 128;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int tl = wn * 128 + j * 32 + (lane & 31);
+        const int tc = tok0 + (tl < tok_rows ? tl : tok_rows - 1);
+        const int64_t tg = a.targets[tc];
+        const bool live = tl < tok_rows && !(a.use_ignore && tg == a.ignore_index);
+        const float gs = live ? a.grad[tc] * gscale : 0.f;
+        const float nlse2 = -a.lse[tc] * kLog2e;
+        // register index (i*16 + r) of the target row in this lane, or -1
+        const int64_t trel = tg - a.v_global0 - vw;
+        const int tr = (trel >= 0 && trel < 128) ? static_cast<int>(trel) : -1;
+        const int x = tr & 31;
+        const int etgt = (tr >= 0 && ((x >> 2) & 1) == (lane >> 5))
+                             ? ((tr >> 5) * 16 + (x >> 3) * 4 + (x & 3))
+                             : -1;
+        uint16_t* drow = a.dz + static_cast<int64_t>(tok0 + tl) * a.ldz + vw + 4 * (lane >> 5);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t o[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int r = q * 4 + c;
+                    float z = acc[i][j][r];
+                    float p;
+                    if (GENERAL) {
+                        const int v = vw + i * 32 + acc_row(r, lane);
+                        if (a.bias != nullptr) z += a.bias[v < a.v_valid ? v : a.v_valid - 1];
+                        p = v < a.v_valid ? __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2)) : 0.f;
+                    } else {
+                        p = __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2));
+                    }
+                    const float hit = (etgt == i * 16 + r) ? gs : 0.f;
+                    o[c] = T::from_float(fmaf(-gs, p, hit));
+                }
+                u32x2_t pk{o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
+                *reinterpret_cast<u32x2_t*>(drow + i * 32 + 8 * q) = pk;
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------- //
+// Backward step 2: dH[tok][h] (+)= sum_v dZ[tok][v] W[v][h]      (M = h, N = token, K = vocab)
+// ------------------------------------------------------------------------------------------- //
+struct DhArgs {
+    const uint16_t* dz;      // [tok_tiles*256][ldz]
+    const uint16_t* weight;  // piece origin [v][H]
+    const float* scales;     // [1] = 1 / loss_scale
+    float* acc;              // fp32 partial dH of the chunk [tok_tiles*256][H] (may be null if single)
+    uint16_t* out;           // dH chunk origin [tok][H], written when `last`
+    int64_t ldz;
+    int H;
+    int v_valid;
+    int tok_valid;
+    int tok_tiles;
+    int h_tiles;
+    int first;  // 1: do not read acc
+    int last;   // 1: write the 16-bit output instead of acc
+};
+
+template <class T, int BK>
+__global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
+{
+    constexpr int TM = 4, TN = 4;
+    using Gemm = TileGemm<T, true, false, TM, TN, BK>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    int tt, ht;
+    xcd_tile(blockIdx.x, a.tok_tiles * a.h_tiles, a.tok_tiles, a.h_tiles, 8, tt, ht);
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int tok0 = tt * 256, h0 = ht * 256;
+
+    Operand A{a.weight + h0, a.H, min(256, a.H - h0)};
+    Operand B{a.dz + static_cast<int64_t>(tok0) * a.ldz, a.ldz, 256};
+    f32x16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    Gemm::run(A, B, a.v_valid, acc, smem);
+
+    const float oscale = a.scales[1];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int tl = tok0 + wn * 128 + j * 32 + (lane & 31);
+        if (tl >= a.tok_valid) continue;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int h = h0 + wm * 128 + i * 32 + 8 * q + 4 * (lane >> 5);
+                if (h >= a.H) continue;  // H % 8 == 0: the quad is all-in or all-out
+                f32x4_t v{acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                          acc[i][j][q * 4 + 3]};
+                float* ap = a.acc + static_cast<int64_t>(tl) * a.H + h;
+                if (!a.first) {
+                    const f32x4_t old = *reinterpret_cast<const f32x4_t*>(ap);
+                    v += old;
+                }
+                if (a.last) {
+                    u32x2_t pk{static_cast<uint32_t>(T::from_float(v.x * oscale)) |
+                                   (static_cast<uint32_t>(T::from_float(v.y * oscale)) << 16),
+                               static_cast<uint32_t>(T::from_float(v.z * oscale)) |
+                                   (static_cast<uint32_t>(T::from_float(v.w * oscale)) << 16)};
+                    *reinterpret_cast<u32x2_t*>(a.out + static_cast<int64_t>(tl) * a.H + h) = pk;
+                } else {
+                    *reinterpret_cast<f32x4_t*>(ap) = v;
+                }
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------- //
+// Backward step 3: dW[v][h] (+)= sum_tok dZ[tok][v] hidden[tok][h]   (M = vocab, N = h, K = token)
+// ------------------------------------------------------------------------------------------- //
+struct DwArgs {
+    const uint16_t* dz;      // [tok_tiles*256][ldz]
+    const uint16_t* hidden;  // chunk origin [tok][H]
+    const float* scales;     // [1] = 1 / loss_scale
+    float* dw;               // piece origin [v][H] fp32
+    int64_t ldz;
+    int H;
+    int v_valid;
+    int tok_valid;
+    int v_tiles;
+    int h_tiles;
+    int accumulate;  // 1: dw += ..., 0: dw = ...
+};
+
+template <class T, int BK>
+__global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
+{
+    constexpr int TM = 4, TN = 4;
+    using Gemm = TileGemm<T, true, true, TM, TN, BK>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    int vt, ht;
+    xcd_tile(blockIdx.x, a.v_tiles * a.h_tiles, a.v_tiles, a.h_tiles, 8, vt, ht);
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int v0 = vt * 256, h0 = ht * 256;
+
+    Operand A{a.dz + v0, a.ldz, 256};
+    Operand B{a.hidden + h0, a.H, min(256, a.H - h0)};
+    f32x16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    Gemm::run(A, B, a.tok_valid, acc, smem);
+
+    const float oscale = a.scales[1];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int h = h0 + wn * 128 + j * 32 + (lane & 31);
+        if (h >= a.H) continue;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int v = v0 + wm * 128 + i * 32 + acc_row(r, lane);
+                if (v >= a.v_valid) continue;
+                float* p = a.dw + static_cast<int64_t>(v) * a.H + h;
+                float val = acc[i][j][r] * oscale;
+                if (a.accumulate) val += *p;
+                *p = val;
+            }
+    }
+}
+
+// db[v] (+)= sum_tok dZ[tok][v], tokens in ascending order (fixed order).
+__global__ void linear_logp_db_kernel(const uint16_t* dz, int64_t ldz, int tok_valid, int v_valid,
+                                      const float* scales, float* db, int accumulate, int dtype)
+{
+    const int v = blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= v_valid) return;
+    float sum = 0.f;
+    for (int t = 0; t < tok_valid; ++t) {
+        const uint16_t x = dz[static_cast<int64_t>(t) * ldz + v];
+        sum += dtype == 0 ? Bf16::to_float(x) : F16::to_float(x);
+    }
+    sum *= scales[1];
+    db[v] = accumulate ? db[v] + sum : sum;
+}
+
+// scales[0] = loss_scale / T, scales[1] = 1 / loss_scale.  For f16 the loss scale is the power of
+// two that brings max|g|/T to about 2^12 so that tiny probabilities survive the f16 dZ; bf16 uses 1.
+__global__ void linear_logp_scales_kernel(const float* grad, int n, float inv_temperature,
+                                          int dtype, float* scales)
+{
+    __shared__ float red[1024];
+    float mx = 0.f;
+    if (dtype == 1) {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) {
+            const float g = fabsf(grad[i]);
+            if (g == g && g != INFINITY) mx = fmaxf(mx, g);
+        }
+    }
+    red[threadIdx.x] = mx;
+    __syncthreads();
+    for (int o = blockDim.x / 2; o > 0; o >>= 1) {
+        if (threadIdx.x < o) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + o]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        float ls = 1.f;
+        if (dtype == 1) {
+            const float top = red[0] * inv_temperature;
+            if (top > 0.f) {
+                int e;
+                frexpf(top, &e);  // top = f * 2^e, f in [0.5, 1)
+                int shift = 12 - e;
+                shift = shift < -24 ? -24 : (shift > 60 ? 60 : shift);
+                ls = ldexpf(1.f, shift);
+            }
+        }
+        scales[0] = ls * inv_temperature;
+        scales[1] = 1.f / ls;
+    }
+}
+
+// Hardware-contract self test of the transposing LDS read used for K-major operands: a 16 x 256
+// tile T[k][r] = k*256 + r is read exactly as TileIO<true,...>::frag does; out[l*8 + e] must equal
+// T[8*(l/32) + e][l % 32] (the MFMA operand layout).
+__global__ void selftest_transpose_read_kernel(int32_t* out)
+{
+    using IO = TileIO<true, 256, 16>;
+    __shared__ __attribute__((aligned(16))) char lds[IO::G::kBytes];
+    for (int i = threadIdx.x; i < 16 * 256; i += 64) {
+        const int k = i / 256, r = i % 256;
+        *reinterpret_cast<uint16_t*>(lds + k * IO::G::kPitch + r * 2) = static_cast<uint16_t>(k * 256 + r);
+    }
+    __syncthreads();
+    const u32x4_t f = IO::frag(lds, 0, 0);
+    const int l = threadIdx.x;
+    const uint32_t w[4] = {f.x, f.y, f.z, f.w};
+    for (int e = 0; e < 8; ++e) out[l * 8 + e] = (w[e >> 1] >> (16 * (e & 1))) & 0xffff;
+}
+
+}  // namespace rlk
+
+// ------------------------------------------------------------------------------------------- //
+// C ABI
+// ------------------------------------------------------------------------------------------- //
+using namespace rlk;
+
+namespace {
+
+constexpr int kBK = RLK_BK;
+
+// Forward launch plan: a pure function of (N, V, bias present).
+//   fast launch   : full vocab tiles [0, full_tiles) split n_fast ways, no bias
+//   general launch: the remaining tiles (all tiles when there is a bias) split n_gen ways
+struct FwdPlan {
+    int row_blocks;
+    int fast_tiles, n_fast;
+    int gen_tiles, n_gen;
+    int total_splits;
+};
+
+int split_count(int row_blocks, int tiles)
+{
+    if (tiles <= 0) return 0;
+    int s = (512 + row_blocks / 2) / row_blocks;
+    if (s < 1) s = 1;
+    if (s > 64) s = 64;
+    if (s > tiles) s = tiles;
+    return s;
+}
+
+FwdPlan fwd_plan(int64_t N, int64_t V, bool has_bias)
+{
+    FwdPlan p;
+    p.row_blocks = static_cast<int>((N + 255) / 256);
+    const int all = static_cast<int>((V + 255) / 256);
+    const int full = static_cast<int>(V / 256);
+    p.fast_tiles = has_bias ? 0 : full;
+    p.gen_tiles = all - p.fast_tiles;
+    p.n_fast = split_count(p.row_blocks, p.fast_tiles);
+    p.n_gen = split_count(p.row_blocks, p.gen_tiles);
+    p.total_splits = p.n_fast + p.n_gen;
+    return p;
+}
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct BwdPlan {
+    int tok_chunk;   // tokens per chunk (multiple of 256)
+    int v_piece;     // vocab rows per piece (multiple of 256)
+    int n_chunks;
+    int n_pieces;
+    size_t dz_bytes;
+    size_t acc_bytes;
+    size_t scales_off, dz_off, acc_off, total;
+};
+
+// Balanced token chunks / vocab pieces so that one dZ block stays within `budget` bytes.
+BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
+{
+    BwdPlan p;
+    const int64_t n_t = (N + 255) / 256, v_t = (V + 255) / 256;
+    // square-ish block: side (in tiles) so that side^2 * 256*256*2 <= budget
+    int64_t side = 1;
+    while ((side + 1) * (side + 1) * 131072 <= static_cast<int64_t>(budget)) ++side;
+    int64_t ct = n_t < side ? n_t : side;
+    int64_t pt = static_cast<int64_t>(budget) / (ct * 131072);
+    if (pt > v_t) pt = v_t;
+    if (pt < 1) pt = 1;
+    p.n_chunks = static_cast<int>((n_t + ct - 1) / ct);
+    p.n_pieces = static_cast<int>((v_t + pt - 1) / pt);
+    p.tok_chunk = static_cast<int>((n_t + p.n_chunks - 1) / p.n_chunks) * 256;
+    p.v_piece = static_cast<int>((v_t + p.n_pieces - 1) / p.n_pieces) * 256;
+    p.dz_bytes = static_cast<size_t>(p.tok_chunk) * p.v_piece * 2;
+    p.acc_bytes = p.n_pieces > 1 ? static_cast<size_t>(p.tok_chunk) * H * 4 : 0;
+    p.scales_off = 0;
+    p.dz_off = 256;
+    p.acc_off = p.dz_off + align_up(p.dz_bytes, 256);
+    p.total = p.acc_off + align_up(p.acc_bytes, 256);
+    return p;
+}
+
+template <class K>
+int set_smem(K kernel, int bytes)
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    return e == hipSuccess ? 0 : rlk_fail(RLK_ERR_LAUNCH, hipGetErrorString(e));
+}
+
+int check_launch(const char* what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, what);
+    return 0;
+}
+
+int check_common(const void* hidden, const void* weight, int64_t N, int32_t H, int64_t V, int dtype)
+{
+    if (dtype != RLK_DTYPE_BF16 && dtype != RLK_DTYPE_F16)
+        return rlk_fail(RLK_ERR_UNSUPPORTED, "dtype must be RLK_DTYPE_BF16 or RLK_DTYPE_F16");
+    if (N <= 0 || H <= 0 || V <= 0) return rlk_fail(RLK_ERR_ARG, "N, H and V must be positive");
+    if (H % 8 != 0) return rlk_fail(RLK_ERR_UNSUPPORTED, "H must be a multiple of 8");
+    if (N > 0x7fff0000LL || V > 0x7fff0000LL) return rlk_fail(RLK_ERR_ARG, "N or V too large");
+    if ((reinterpret_cast<uintptr_t>(hidden) & 15) || (reinterpret_cast<uintptr_t>(weight) & 15))
+        return rlk_fail(RLK_ERR_ARG, "hidden and weight must be 16-byte aligned");
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rlk_linear_logp_fwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                                        size_t* bytes)
+{
+    (void)H;
+    (void)dtype;
+    if (!bytes || N <= 0 || V <= 0) return rlk_fail(RLK_ERR_ARG, "bad workspace query");
+    // sized for the larger of the two plans so that one query serves calls with and without bias
+    const int a = fwd_plan(N, V, false).total_splits, b = fwd_plan(N, V, true).total_splits;
+    *bytes = static_cast<size_t>(3) * (a > b ? a : b) * N * sizeof(float);
+    return 0;
+}
+
+int rlk_linear_logp_fwd(const void* hidden, const void* weight, const float* bias,
+                        const int64_t* targets, float* logp, float* lse, void* workspace,
+                        size_t workspace_bytes, int64_t N, int32_t H, int64_t V,
+                        int64_t vocab_start, int32_t dtype, float temperature,
+                        int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
+                        int32_t* err_flag, hipStream_t stream)
+{
+    if (int rc = check_common(hidden, weight, N, H, V, dtype)) return rc;
+    if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
+    if (!targets || !logp || !lse || !err_flag) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    size_t need = 0;
+    rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &need);
+    if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
+
+    FwdArgs a;
+    a.hidden = static_cast<const uint16_t*>(hidden);
+    a.weight = static_cast<const uint16_t*>(weight);
+    a.bias = bias;
+    a.targets = targets;
+    a.N = static_cast<int>(N);
+    a.H = H;
+    a.V = static_cast<int>(V);
+    a.vocab_start = vocab_start;
+    const FwdPlan plan = fwd_plan(N, V, bias != nullptr);
+    a.row_blocks = plan.row_blocks;
+    a.part_m = static_cast<float*>(workspace);
+    a.part_s = a.part_m + static_cast<size_t>(plan.total_splits) * N;
+    a.part_z = a.part_s + static_cast<size_t>(plan.total_splits) * N;
+    a.scale2 = kLog2e / temperature;
+
+    using G = TileGemm<Bf16, false, false, 4, 4, kBK>;  // same LDS footprint for f16
+    if (plan.n_fast > 0) {
+        a.n_split = plan.n_fast;
+        a.split_lo = 0;
+        a.tile_lo = 0;
+        a.vtiles = plan.fast_tiles;
+        const int grid = a.row_blocks * a.n_split;
+        if (dtype == RLK_DTYPE_BF16) {
+            if (int rc = set_smem(linear_logp_fwd_kernel<Bf16, kBK, false>, G::kSmemBytes)) return rc;
+            hipLaunchKernelGGL((linear_logp_fwd_kernel<Bf16, kBK, false>), dim3(grid), dim3(kThreads),
+                               G::kSmemBytes, stream, a);
+        } else {
+            if (int rc = set_smem(linear_logp_fwd_kernel<F16, kBK, false>, G::kSmemBytes)) return rc;
+            hipLaunchKernelGGL((linear_logp_fwd_kernel<F16, kBK, false>), dim3(grid), dim3(kThreads),
+                               G::kSmemBytes, stream, a);
+        }
+    }
+    if (plan.n_gen > 0) {
+        a.n_split = plan.n_gen;
+        a.split_lo = plan.n_fast;
+        a.tile_lo = plan.fast_tiles;
+        a.vtiles = plan.gen_tiles;
+        const int grid = a.row_blocks * a.n_split;
+        if (dtype == RLK_DTYPE_BF16) {
+            if (int rc = set_smem(linear_logp_fwd_kernel<Bf16, kBK, true>, G::kSmemBytes)) return rc;
+            hipLaunchKernelGGL((linear_logp_fwd_kernel<Bf16, kBK, true>), dim3(grid), dim3(kThreads),
+                               G::kSmemBytes, stream, a);
+        } else {
+            if (int rc = set_smem(linear_logp_fwd_kernel<F16, kBK, true>, G::kSmemBytes)) return rc;
+            hipLaunchKernelGGL((linear_logp_fwd_kernel<F16, kBK, true>), dim3(grid), dim3(kThreads),
+                               G::kSmemBytes, stream, a);
+        }
+    }
+    if (int rc = check_launch("linear_logp_fwd_kernel launch failed")) return rc;
+
+    CombineArgs c;
+    c.part_m = a.part_m;
+    c.part_s = a.part_s;
+    c.part_z = a.part_z;
+    c.targets = targets;
+    c.logp = logp;
+    c.lse = lse;
+    c.err_flag = err_flag;
+    c.N = a.N;
+    c.V = a.V;
+    c.n_split = plan.total_splits;
+    c.vocab_start = vocab_start;
+    c.ignore_index = ignore_index;
+    c.use_ignore = use_ignore;
+    c.strict = strict_targets;
+    hipLaunchKernelGGL(linear_logp_combine_kernel, dim3((a.N + 255) / 256), dim3(256), 0, stream, c);
+    return check_launch("linear_logp_combine_kernel launch failed");
+}
+
+int rlk_selftest_transpose_read(int32_t* out, hipStream_t stream)
+{
+    if (!out) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    hipLaunchKernelGGL(selftest_transpose_read_kernel, dim3(1), dim3(64), 0, stream, out);
+    return check_launch("selftest launch failed");
+}
+
+int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                                        size_t dz_budget_bytes, size_t* bytes)
+{
+    (void)dtype;
+    if (!bytes || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad workspace query");
+    if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
+    if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
+    *bytes = bwd_plan(N, H, V, dz_budget_bytes).total;
+    return 0;
+}
+
+int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* weight,
+                        const float* bias, const int64_t* targets, const float* lse,
+                        void* d_hidden, float* d_weight, float* d_bias, void* workspace,
+                        size_t workspace_bytes, size_t dz_budget_bytes, int64_t N, int32_t H,
+                        int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                        int64_t ignore_index, int32_t use_ignore, hipStream_t stream)
+{
+    if (int rc = check_common(hidden, weight, N, H, V, dtype)) return rc;
+    if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
+    if (!grad_logp || !targets || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (!d_hidden && !d_weight && !d_bias) return rlk_fail(RLK_ERR_ARG, "no gradient requested");
+    if (bias == nullptr && d_bias != nullptr) return rlk_fail(RLK_ERR_ARG, "d_bias given without bias");
+    if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
+    if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
+    const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
+    if (!workspace || workspace_bytes < p.total) return rlk_fail(RLK_ERR_ARG, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(workspace) & 255)
+        return rlk_fail(RLK_ERR_ARG, "workspace must be 256-byte aligned");
+
+    char* ws = static_cast<char*>(workspace);
+    float* scales = reinterpret_cast<float*>(ws + p.scales_off);
+    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.dz_off);
+    float* hacc = p.acc_bytes ? reinterpret_cast<float*>(ws + p.acc_off) : nullptr;
+    const uint16_t* hid = static_cast<const uint16_t*>(hidden);
+    const uint16_t* w = static_cast<const uint16_t*>(weight);
+    uint16_t* dh = static_cast<uint16_t*>(d_hidden);
+    const int h_tiles = (H + 255) / 256;
+
+    hipLaunchKernelGGL(linear_logp_scales_kernel, dim3(1), dim3(1024), 0, stream, grad_logp,
+                       static_cast<int>(N), 1.f / temperature, dtype, scales);
+    if (int rc = check_launch("scales kernel launch failed")) return rc;
+
+    using GZb = TileGemm<Bf16, false, false, 4, 4, kBK>;
+    using GHb = TileGemm<Bf16, true, false, 4, 4, kBK>;
+    using GWb = TileGemm<Bf16, true, true, 4, 4, kBK>;
+    if (dtype == RLK_DTYPE_BF16) {
+        if (int rc = set_smem(linear_logp_dz_kernel<Bf16, kBK, false>, GZb::kSmemBytes)) return rc;
+        if (int rc = set_smem(linear_logp_dz_kernel<Bf16, kBK, true>, GZb::kSmemBytes)) return rc;
+        if (int rc = set_smem(linear_logp_dh_kernel<Bf16, kBK>, GHb::kSmemBytes)) return rc;
+        if (int rc = set_smem(linear_logp_dw_kernel<Bf16, kBK>, GWb::kSmemBytes)) return rc;
+    } else {
+        if (int rc = set_smem(linear_logp_dz_kernel<F16, kBK, false>, GZb::kSmemBytes)) return rc;
+        if (int rc = set_smem(linear_logp_dz_kernel<F16, kBK, true>, GZb::kSmemBytes)) return rc;
+        if (int rc = set_smem(linear_logp_dh_kernel<F16, kBK>, GHb::kSmemBytes)) return rc;
+        if (int rc = set_smem(linear_logp_dw_kernel<F16, kBK>, GWb::kSmemBytes)) return rc;
+    }
+
+    for (int ci = 0; ci < p.n_chunks; ++ci) {
+        const int64_t tok_lo = static_cast<int64_t>(ci) * p.tok_chunk;
+        const int tok_valid = static_cast<int>((N - tok_lo) < p.tok_chunk ? (N - tok_lo) : p.tok_chunk);
+        if (tok_valid <= 0) break;
+        const int tok_tiles = (tok_valid + 255) / 256;
+        for (int pi = 0; pi < p.n_pieces; ++pi) {
+            const int64_t v_lo = static_cast<int64_t>(pi) * p.v_piece;
+            const int v_valid = static_cast<int>((V - v_lo) < p.v_piece ? (V - v_lo) : p.v_piece);
+            if (v_valid <= 0) break;
+            const int v_tiles = (v_valid + 255) / 256;
+            const bool last_piece = (v_lo + p.v_piece >= V);
+
+            DzArgs z;
+            z.hidden = hid + tok_lo * H;
+            z.weight = w + v_lo * H;
+            z.bias = bias ? bias + v_lo : nullptr;
+            z.targets = targets + tok_lo;
+            z.lse = lse + tok_lo;
+            z.grad = grad_logp + tok_lo;
+            z.scales = scales;
+            z.dz = dz;
+            z.ldz = p.v_piece;
+            z.tok_valid = tok_valid;
+            z.v_valid = v_valid;
+            z.H = H;
+            z.tok_tiles = tok_tiles;
+            z.v_global0 = vocab_start + v_lo;
+            z.ignore_index = ignore_index;
+            z.use_ignore = use_ignore;
+            z.scale2 = kLog2e / temperature;
+
+            DhArgs h;
+            h.dz = dz;
+            h.weight = w + v_lo * H;
+            h.scales = scales;
+            h.acc = hacc;
+            h.out = dh ? dh + tok_lo * H : nullptr;
+            h.ldz = p.v_piece;
+            h.H = H;
+            h.v_valid = v_valid;
+            h.tok_valid = tok_valid;
+            h.tok_tiles = tok_tiles;
+            h.h_tiles = h_tiles;
+            h.first = pi == 0;
+            h.last = last_piece;
+
+            DwArgs d;
+            d.dz = dz;
+            d.hidden = hid + tok_lo * H;
+            d.scales = scales;
+            d.dw = d_weight ? d_weight + v_lo * H : nullptr;
+            d.ldz = p.v_piece;
+            d.H = H;
+            d.v_valid = v_valid;
+            d.tok_valid = tok_valid;
+            d.v_tiles = v_tiles;
+            d.h_tiles = h_tiles;
+            d.accumulate = ci > 0;
+
+            // dZ block: full vocab tiles through the fast variant, the rest (all of them when
+            // there is a bias) through the general one
+            const int fast_tiles = bias ? 0 : v_valid / 256;
+            const int gen_tiles = v_tiles - fast_tiles;
+            if (dtype == RLK_DTYPE_BF16) {
+                if (fast_tiles > 0) {
+                    z.v_tiles = fast_tiles;
+                    z.v_tile_lo = 0;
+                    hipLaunchKernelGGL((linear_logp_dz_kernel<Bf16, kBK, false>),
+                                       dim3(tok_tiles * fast_tiles), dim3(kThreads), GZb::kSmemBytes,
+                                       stream, z);
+                }
+                if (gen_tiles > 0) {
+                    z.v_tiles = gen_tiles;
+                    z.v_tile_lo = fast_tiles;
+                    hipLaunchKernelGGL((linear_logp_dz_kernel<Bf16, kBK, true>),
+                                       dim3(tok_tiles * gen_tiles), dim3(kThreads), GZb::kSmemBytes,
+                                       stream, z);
+                }
+                if (d_hidden)
+                    hipLaunchKernelGGL((linear_logp_dh_kernel<Bf16, kBK>), dim3(tok_tiles * h_tiles),
+                                       dim3(kThreads), GHb::kSmemBytes, stream, h);
+                if (d_weight)
+                    hipLaunchKernelGGL((linear_logp_dw_kernel<Bf16, kBK>), dim3(v_tiles * h_tiles),
+                                       dim3(kThreads), GWb::kSmemBytes, stream, d);
+            } else {
+                if (fast_tiles > 0) {
+                    z.v_tiles = fast_tiles;
+                    z.v_tile_lo = 0;
+                    hipLaunchKernelGGL((linear_logp_dz_kernel<F16, kBK, false>),
+                                       dim3(tok_tiles * fast_tiles), dim3(kThreads), GZb::kSmemBytes,
+                                       stream, z);
+                }
+                if (gen_tiles > 0) {
+                    z.v_tiles = gen_tiles;
+                    z.v_tile_lo = fast_tiles;
+                    hipLaunchKernelGGL((linear_logp_dz_kernel<F16, kBK, true>),
+                                       dim3(tok_tiles * gen_tiles), dim3(kThreads), GZb::kSmemBytes,
+                                       stream, z);
+                }
+                if (d_hidden)
+                    hipLaunchKernelGGL((linear_logp_dh_kernel<F16, kBK>), dim3(tok_tiles * h_tiles),
+                                       dim3(kThreads), GHb::kSmemBytes, stream, h);
+                if (d_weight)
+                    hipLaunchKernelGGL((linear_logp_dw_kernel<F16, kBK>), dim3(v_tiles * h_tiles),
+                                       dim3(kThreads), GWb::kSmemBytes, stream, d);
+            }
+            if (d_bias != nullptr) {
+                hipLaunchKernelGGL(linear_logp_db_kernel, dim3((v_valid + 255) / 256), dim3(256), 0,
+                                   stream, dz, static_cast<int64_t>(p.v_piece), tok_valid, v_valid,
+                                   scales, d_bias + v_lo, ci > 0 ? 1 : 0, dtype);
+            }
+            if (int rc = check_launch("linear_logp backward launch failed")) return rc;
+        }
+    }
+    return 0;
+}
+
+}  // extern "C"

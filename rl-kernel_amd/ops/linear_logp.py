@@ -1,0 +1,245 @@
+"""Fused linear -> selected-token log-prob on MI355X.
+
+``RocmFusedLinearLogpOp`` has the call signature of the reference's ``linear_logp`` backends
+(rl_engine/kernels/ops/pytorch/loss/linear_logp.py:455-486,
+rl_engine/kernels/ops/cuda/loss/linear_logp.py:252-359) and is differentiable w.r.t. hidden,
+weight and bias.  Two keyword-only extensions with neutral defaults fold the caller-side
+conventions of rl_engine/testing/reference_ops.py:15-47 into the kernel: ``temperature`` and
+``ignore_index``.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+
+from .. import _native
+from ..platform import logger
+
+_DTYPES = {torch.bfloat16: _native.DTYPE_BF16, torch.float16: _native.DTYPE_F16}
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _aligned_contiguous(t: torch.Tensor) -> torch.Tensor:
+    t = t.contiguous()
+    if t.data_ptr() % 16:
+        t = t.clone(memory_format=torch.contiguous_format)
+    return t
+
+
+def _out_of_range_error(target_1d: torch.Tensor, vocab: int, ignore_index: Optional[int]):
+    live = target_1d if ignore_index is None else target_1d[target_1d != ignore_index]
+    t_min, t_max = int(live.min()), int(live.max())
+    return ValueError(
+        f"target_ids out of range: expected [0, {vocab - 1}], got [{t_min}, {t_max}]. "
+        "Mask or filter padding / ignore-index values (e.g. -100) before this op."
+    )
+
+
+def mfma_path_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
+    """bf16/f16 on the GPU with a hidden size the 16-byte tile loads can address."""
+    return (
+        hidden.is_cuda
+        and weight.is_cuda
+        and hidden.device == weight.device
+        and hidden.dtype in _DTYPES
+        and weight.dtype == hidden.dtype
+        and hidden.size(-1) % 8 == 0
+    )
+
+
+def fused_linear_logp_forward(
+    hidden_2d: torch.Tensor,
+    weight: torch.Tensor,
+    target_1d: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    *,
+    temperature: float = 1.0,
+    ignore_index: Optional[int] = None,
+    vocab_start: int = 0,
+    strict_targets: bool = True,
+):
+    """Raw forward: returns ``(logp, lse, err_flag)`` fp32 / fp32 / int32[1] device tensors.
+
+    Stand-in for ``_C.fused_linear_logp_sm90`` (csrc/cuda/fused_linear_logp_sm90.cu:305-381 of the
+    reference) with int64 global targets.  Does not synchronise; ``err_flag`` is non-zero when
+    ``strict_targets`` and some non-ignored target lies outside the weight shard.
+    """
+    lib = _native.load()
+    n, h = hidden_2d.shape
+    v = weight.size(0)
+    dev = hidden_2d.device
+    logp = torch.empty(n, device=dev, dtype=torch.float32)
+    lse = torch.empty(n, device=dev, dtype=torch.float32)
+    err = torch.zeros(1, device=dev, dtype=torch.int32)
+    need = _native.ctypes.c_size_t(0)
+    dt = _DTYPES[hidden_2d.dtype]
+    _native.check(lib.rlk_linear_logp_fwd_workspace_bytes(n, h, v, dt, _native.ctypes.byref(need)),
+                  "linear_logp workspace query")
+    ws = torch.empty(max(need.value, 16), device=dev, dtype=torch.uint8)
+    bias_f = None if bias is None else bias.detach().to(torch.float32).contiguous()
+    rc = lib.rlk_linear_logp_fwd(
+        _ptr(hidden_2d), _ptr(weight), _ptr(bias_f), _ptr(target_1d), _ptr(logp), _ptr(lse),
+        _ptr(ws), ws.numel(), n, h, v, int(vocab_start), dt, float(temperature),
+        0 if ignore_index is None else int(ignore_index), int(ignore_index is not None),
+        int(strict_targets), _ptr(err), _stream(dev))
+    _native.check(rc, "rlk_linear_logp_fwd")
+    return logp, lse, err
+
+
+def fused_linear_logp_backward(
+    grad_logp: torch.Tensor,
+    hidden_2d: torch.Tensor,
+    weight: torch.Tensor,
+    target_1d: torch.Tensor,
+    lse: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    *,
+    temperature: float = 1.0,
+    ignore_index: Optional[int] = None,
+    vocab_start: int = 0,
+    need_hidden: bool = True,
+    need_weight: bool = True,
+    need_bias: bool = True,
+    dz_budget_bytes: int = 0,
+):
+    """Raw backward: ``(d_hidden [N,H] input dtype, d_weight [V,H] fp32, d_bias [V] fp32)``.
+
+    Stand-in for ``chunked_linear_logp_backward``
+    (rl_engine/kernels/ops/pytorch/loss/linear_logp.py:383-439 of the reference); unlike it, the
+    saved ``lse`` is used (as the vocab-parallel backward does, :313).
+    """
+    lib = _native.load()
+    n, h = hidden_2d.shape
+    v = weight.size(0)
+    dev = hidden_2d.device
+    dt = _DTYPES[hidden_2d.dtype]
+    g = grad_logp.reshape(-1).to(torch.float32).contiguous()
+    d_hidden = torch.empty_like(hidden_2d) if need_hidden else None
+    d_weight = torch.empty(v, h, device=dev, dtype=torch.float32) if need_weight else None
+    want_bias = bias is not None and need_bias
+    d_bias = torch.empty(v, device=dev, dtype=torch.float32) if want_bias else None
+    bias_f = None if bias is None else bias.detach().to(torch.float32).contiguous()
+    need = _native.ctypes.c_size_t(0)
+    _native.check(lib.rlk_linear_logp_bwd_workspace_bytes(n, h, v, dt, int(dz_budget_bytes),
+                                                          _native.ctypes.byref(need)),
+                  "linear_logp backward workspace query")
+    ws = torch.empty(need.value, device=dev, dtype=torch.uint8)
+    rc = lib.rlk_linear_logp_bwd(
+        _ptr(g), _ptr(hidden_2d), _ptr(weight), _ptr(bias_f), _ptr(target_1d), _ptr(lse),
+        _ptr(d_hidden), _ptr(d_weight), _ptr(d_bias), _ptr(ws), ws.numel(), int(dz_budget_bytes),
+        n, h, v, int(vocab_start), dt, float(temperature),
+        0 if ignore_index is None else int(ignore_index), int(ignore_index is not None),
+        _stream(dev))
+    _native.check(rc, "rlk_linear_logp_bwd")
+    return d_hidden, d_weight, d_bias
+
+
+class _FusedLinearLogpFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, weight, bias, target_ids, temperature, ignore_index, check_targets):
+        hidden_2d = _aligned_contiguous(hidden.reshape(-1, hidden.size(-1)))
+        w = _aligned_contiguous(weight)
+        target_1d = target_ids.reshape(-1).to(device=hidden_2d.device, dtype=torch.long).contiguous()
+        logp, lse, err = fused_linear_logp_forward(
+            hidden_2d, w, target_1d, bias, temperature=temperature, ignore_index=ignore_index)
+        if check_targets and bool(err.item()):
+            raise _out_of_range_error(target_1d, w.size(0), ignore_index)
+        ctx.save_for_backward(hidden_2d, w, bias if bias is not None else hidden_2d, target_1d, lse)
+        ctx.has_bias = bias is not None
+        ctx.lead_shape = hidden.shape[:-1]
+        ctx.temperature = temperature
+        ctx.ignore_index = ignore_index
+        ctx.weight_dtype = weight.dtype
+        ctx.bias_dtype = bias.dtype if bias is not None else None
+        return logp.reshape(hidden.shape[:-1])
+
+    @staticmethod
+    def backward(ctx, grad_logp):
+        hidden_2d, w, bias_t, target_1d, lse = ctx.saved_tensors
+        need_h, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[1], \
+            ctx.has_bias and ctx.needs_input_grad[2]
+        d_h, d_w, d_b = fused_linear_logp_backward(
+            grad_logp, hidden_2d, w, target_1d, lse, bias_t if ctx.has_bias else None,
+            temperature=ctx.temperature, ignore_index=ctx.ignore_index,
+            need_hidden=need_h, need_weight=need_w, need_bias=need_b)
+        grad_hidden = d_h.reshape(tuple(ctx.lead_shape) + (hidden_2d.size(1),)) if need_h else None
+        grad_weight = d_w.to(ctx.weight_dtype) if need_w else None
+        grad_bias = d_b.to(ctx.bias_dtype) if need_b else None
+        return grad_hidden, grad_weight, grad_bias, None, None, None, None
+
+
+class RocmFusedLinearLogpOp:
+    """gfx950 MFMA fused linear log-prob: ``log_softmax((hidden W^T + b)/T)[target]`` without the
+    ``[N, V]`` logits.  Constructor raises ``RuntimeError`` when the HIP library or a ROCm GPU is
+    missing so that a registry can fall through to its next backend
+    (rl_engine/kernels/registry.py:219-229 of the reference)."""
+
+    def __init__(self) -> None:
+        if not torch.cuda.is_available() or getattr(torch.version, "hip", None) is None:
+            raise RuntimeError("RocmFusedLinearLogpOp needs a ROCm GPU")
+        _native.load()
+        logger.info("Linked to librlk_hip.so fused linear_logp kernels.")
+
+    def __call__(self, hidden, lm_head_weight, target_ids, bias=None, *, tp_group: Any = None,
+                 vocab_start_index: int = 0, global_vocab_size: Optional[int] = None,
+                 temperature: float = 1.0, ignore_index: Optional[int] = None,
+                 check_targets: bool = True) -> torch.Tensor:
+        return self.apply(hidden, lm_head_weight, target_ids, bias, tp_group=tp_group,
+                          vocab_start_index=vocab_start_index, global_vocab_size=global_vocab_size,
+                          temperature=temperature, ignore_index=ignore_index,
+                          check_targets=check_targets)
+
+    def apply(self, hidden, lm_head_weight, target_ids, bias=None, *, tp_group: Any = None,
+              vocab_start_index: int = 0, global_vocab_size: Optional[int] = None,
+              temperature: float = 1.0, ignore_index: Optional[int] = None,
+              check_targets: bool = True) -> torch.Tensor:
+        """Selected-token log-prob in float32 with the leading shape of ``hidden``."""
+        if temperature <= 0.0:
+            raise ValueError("temperature must be greater than zero")
+        if lm_head_weight.size(-1) != hidden.size(-1):
+            raise ValueError(
+                f"hidden dim {hidden.size(-1)} must match lm_head_weight dim "
+                f"{lm_head_weight.size(-1)}")
+        if lm_head_weight.device != hidden.device:
+            raise ValueError(
+                f"lm_head_weight device {lm_head_weight.device} must match hidden "
+                f"device {hidden.device}")
+        if hidden.shape[:-1] != target_ids.shape:
+            raise ValueError(
+                f"hidden leading shape {tuple(hidden.shape[:-1])} must match "
+                f"target_ids shape {tuple(target_ids.shape)}")
+        vocab = lm_head_weight.size(0)
+        if bias is not None:
+            if bias.ndim != 1 or bias.numel() != vocab:
+                raise ValueError(f"bias must be 1-D with V={vocab} elements, got "
+                                 f"shape {tuple(bias.shape)}")
+            if bias.device != hidden.device:
+                raise ValueError(f"bias device {bias.device} must match hidden device "
+                                 f"{hidden.device}")
+        # Vocab-parallel metadata follows the reference's argument policy
+        # (rl_engine/kernels/ops/pytorch/loss/linear_logp.py:58-83): without a multi-rank group it
+        # is an error.  This build runs on one GPU; a multi-rank group is not implemented.
+        if vocab <= 0:
+            raise ValueError("lm_head_weight must contain at least one vocab row.")
+        if tp_group is not None:
+            raise NotImplementedError(
+                "vocab-parallel linear_logp over a process group is not part of the one-GPU build")
+        if vocab_start_index != 0:
+            raise ValueError("vocab_start_index requires a tensor-parallel group.")
+        if global_vocab_size is not None and int(global_vocab_size) != vocab:
+            raise ValueError("global_vocab_size differs from the local vocab size, but no "
+                             "multi-rank tensor-parallel group was provided.")
+        if not mfma_path_supported(hidden, lm_head_weight):
+            raise NotImplementedError(
+                "RocmFusedLinearLogpOp: needs bf16/f16 CUDA tensors with hidden size % 8 == 0")
+        return _FusedLinearLogpFunction.apply(hidden, lm_head_weight, bias, target_ids,
+                                              float(temperature), ignore_index, check_targets)
