@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused linear-logprob hot path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+One step = one forward (logp, lse) + one backward (dH in the input dtype, dW fp32) of the fused
+LM-head log-prob over one synthetic batch at the Llama-3-8B head shape (32768 tokens, H=4096,
+V=128256, bf16), through the C-ABI library.  Inputs are resident in HBM before the timed region.
+Prints ONE JSON line (metric = tokens/s of the whole step) carrying a `roofline` object for the
+dominant kernel (the forward contraction, timed with HIP events on the launch stream) and a
+`cpu_baseline` object (the CPU oracle timed on a bounded token slice on the host cores).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}  # MI355X dense MFMA, published
+
+WORKLOADS = {
+    # BASELINE.json configs[1] shape; the metric is quoted on forward+backward at this shape
+    "llama3-8b-head": dict(tokens=32768, hidden=4096, vocab=128256, dtype="bf16",
+                           temperature=1.0, ignore_frac=0.0),
+    "llama3-8b-head-64k": dict(tokens=65536, hidden=4096, vocab=128256, dtype="bf16",
+                               temperature=0.7, ignore_frac=0.0),
+    "qwen3-head": dict(tokens=131072, hidden=2048, vocab=151936, dtype="f16",
+                       temperature=1.0, ignore_frac=0.01),
+    "small": dict(tokens=4096, hidden=1024, vocab=32768, dtype="bf16", temperature=1.0,
+                  ignore_frac=0.0),
+}
+
+
+def make_inputs(torch, cfg, device, seed=1002):
+    gen = torch.Generator(device=device).manual_seed(seed)
+    dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float16
+    n, h, v = cfg["tokens"], cfg["hidden"], cfg["vocab"]
+    hidden = torch.randn(n, h, device=device, dtype=torch.float32, generator=gen).to(dt)
+    weight = torch.empty(v, h, device=device, dtype=dt)
+    step = 16384  # generate W in slabs to bound the fp32 temporary
+    for v0 in range(0, v, step):
+        v1 = min(v, v0 + step)
+        weight[v0:v1] = (torch.randn(v1 - v0, h, device=device, dtype=torch.float32,
+                                     generator=gen) * 0.02).to(dt)
+    targets = torch.randint(0, v, (n,), device=device, generator=gen)
+    if cfg["ignore_frac"] > 0:
+        drop = torch.rand(n, device=device, generator=gen) < cfg["ignore_frac"]
+        targets = torch.where(drop, torch.full_like(targets, -100), targets)
+    grad = torch.randn(n, device=device, dtype=torch.float32, generator=gen)
+    return hidden, weight, targets, grad
+
+
+def cpu_baseline(torch, cfg, slice_tokens, iters=3):
+    """Time the CPU oracle (fp32 linear + log_softmax + gather, closed-form backward) on a slice."""
+    from oracle import oracle as O
+
+    gen = torch.Generator().manual_seed(7)
+    h, v = cfg["hidden"], cfg["vocab"]
+    hidden = torch.randn(slice_tokens, h, generator=gen)
+    weight = torch.randn(v, h, generator=gen) * 0.02
+    targets = torch.randint(0, v, (slice_tokens,), generator=gen)
+    grad = torch.randn(slice_tokens, generator=gen)
+
+    def step():
+        O.linear_logp(hidden, weight, targets, temperature=cfg["temperature"])
+        O.linear_logp_backward(grad, hidden, weight, targets, temperature=cfg["temperature"],
+                               token_chunk=1024)
+
+    step()  # warm-up
+    times = []
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": slice_tokens / med,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{slice_tokens}-token slice at the full H={h}, V={v}; fp32 torch CPU oracle "
+                  f"forward+backward, 1 warm-up + {iters} timed, median; host cpu_count="
+                  f"{os.cpu_count()}",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama3-8b-head", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-slice", type=int, default=1024,
+                    help="tokens of the CPU-baseline slice (0 = skip the CPU baseline)")
+    ap.add_argument("--mode", default="fwd+bwd", choices=["fwd+bwd", "fwd"])
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; every figure is a one-GPU figure. "
+              "Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
+        return 3
+
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    cfg = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    hidden, weight, targets, grad = make_inputs(torch, cfg, dev)
+    n, h, v = cfg["tokens"], cfg["hidden"], cfg["vocab"]
+    ign = -100 if cfg["ignore_frac"] > 0 else None
+    temp = cfg["temperature"]
+    do_bwd = args.mode == "fwd+bwd"
+
+    fwd_ev = []
+
+    def step(record=False):
+        if record:
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+        logp, lse, err = LL.fused_linear_logp_forward(hidden, weight, targets, None,
+                                                      temperature=temp, ignore_index=ign)
+        if record:
+            e1.record()
+            fwd_ev.append((e0, e1))
+        out = (logp, lse)
+        if do_bwd:
+            d_h, d_w, _ = LL.fused_linear_logp_backward(grad, hidden, weight, targets, lse, None,
+                                                        temperature=temp, ignore_index=ign)
+            out = (logp, lse, d_h, d_w)
+        return out
+
+    torch.cuda.synchronize()
+    base_mem = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    first = step()
+    torch.cuda.synchronize()
+    out_bytes = sum(t.numel() * t.element_size() for t in first)
+    peak_extra = torch.cuda.max_memory_allocated() - base_mem - out_bytes
+    for _ in range(max(0, args.warmup - 1)):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    last = None
+    for _ in range(args.steps):
+        last = step(record=True)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms = elapsed * 1e3 / args.steps
+
+    deterministic = all(torch.equal(a, b) for a, b in zip(first, last))
+    fwd_ms = sum(a.elapsed_time(b) for a, b in fwd_ev) / len(fwd_ev)
+    fwd_flops = 2.0 * n * h * v
+    achieved = fwd_flops / (fwd_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[cfg["dtype"]]
+    step_flops = (8.0 if do_bwd else 2.0) * n * h * v
+
+    result = {
+        "metric": "logp fwd+bwd tokens/sec" if do_bwd else "logp fwd tokens/sec",
+        "value": n / (ms * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: fused LM-head logp {args.mode}, {n} tokens, H={h}, "
+                        f"V={v}, {cfg['dtype']} in / fp32 accumulate, T={temp}",
+            "tokens": n, "hidden": h, "vocab": v, "mode": args.mode,
+        },
+        "step_tflops": step_flops / (ms * 1e-3) / 1e12,
+        "step_frac_of_mfma_peak": step_flops / (ms * 1e-3) / 1e12 / peak,
+        "step_flop_accounting": "8*N*H*V (fwd 2 + logit recompute 2 + dH 2 + dW 2)" if do_bwd
+                                else "2*N*H*V",
+        "peak_extra_hbm_bytes": int(peak_extra),
+        "bitwise_repeatable": bool(deterministic),
+        "roofline": {
+            "kernel": "linear_logp_fwd_kernel",
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": peak,
+            "unit": "TFLOP/s",
+            "frac": achieved / peak,
+            "traffic": None,
+            "launch_ms": fwd_ms,
+            "flops_per_launch": fwd_flops,
+        },
+    }
+    if args.cpu_slice > 0:
+        result["cpu_baseline"] = cpu_baseline(torch, cfg, args.cpu_slice)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

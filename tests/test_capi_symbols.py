@@ -1,0 +1,91 @@
+"""CPU-side checks of the C-ABI boundary: the library loads, exports every symbol the header
+declares, and its host-only planning entry points behave (no GPU work is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "rlk_hip.h")
+
+
+@pytest.fixture(scope="module")
+def native():
+    from rl_kernel_amd import _native
+
+    if not os.path.exists(_native.LIB_PATH):
+        import importlib
+
+        importlib.import_module("rl_kernel_amd.build").build()
+    return _native
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rlk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_something():
+    names = declared_symbols()
+    assert "rlk_linear_logp_fwd" in names and "rlk_linear_logp_bwd" in names
+
+
+def test_library_exports_every_declared_symbol(native):
+    lib = ctypes.CDLL(native.LIB_PATH)
+    missing = [n for n in declared_symbols() if not hasattr(lib, n)]
+    assert not missing, f"declared in include/rlk_hip.h but not exported: {missing}"
+
+
+def test_binding_covers_every_declared_symbol(native):
+    assert sorted(native.SIGNATURES) == declared_symbols()
+    lib = native.load()
+    assert lib.rlk_version() >= 100
+    assert lib.rlk_last_error() is not None
+
+
+def test_backward_workspace_is_constant_in_token_count(native):
+    lib = native.load()
+    sizes = []
+    for n in (32768, 65536, 131072, 262144):
+        need = ctypes.c_size_t(0)
+        assert lib.rlk_linear_logp_bwd_workspace_bytes(n, 4096, 128256, 0, 0, ctypes.byref(need)) == 0
+        sizes.append(need.value)
+    assert len(set(sizes)) == 1, sizes          # same scratch for G = 64, 128, 256, 512
+    assert sizes[0] <= 1 << 30                  # <= 1 GiB extra HBM
+    need = ctypes.c_size_t(0)
+    assert lib.rlk_linear_logp_bwd_workspace_bytes(131072, 2048, 151936, 1, 0, ctypes.byref(need)) == 0
+    assert need.value <= 1 << 30
+
+
+def test_forward_workspace_is_small(native):
+    lib = native.load()
+    need = ctypes.c_size_t(0)
+    assert lib.rlk_linear_logp_fwd_workspace_bytes(32768, 4096, 128256, 0, ctypes.byref(need)) == 0
+    assert 0 < need.value <= 64 << 20
+
+
+def test_bad_arguments_are_reported_not_launched(native):
+    lib = native.load()
+    need = ctypes.c_size_t(0)
+    assert lib.rlk_linear_logp_fwd_workspace_bytes(0, 4096, 128256, 0, ctypes.byref(need)) == -1
+    assert b"workspace" in lib.rlk_last_error()
+    # null pointers / unsupported dtype are rejected on the host before any launch
+    rc = lib.rlk_linear_logp_fwd(None, None, None, None, None, None, None, 0, 16, 64, 32, 0, 7, 1.0,
+                                 0, 0, 1, None, None)
+    assert rc == -2
+    rc = lib.rlk_linear_logp_fwd(None, None, None, None, None, None, None, 0, 16, 60, 32, 0, 0, 1.0,
+                                 0, 0, 1, None, None)
+    assert rc == -2 and b"multiple of 8" in lib.rlk_last_error()
+    rc = lib.rlk_linear_logp_fwd(None, None, None, None, None, None, None, 0, 16, 64, 32, 0, 0, 0.0,
+                                 0, 0, 1, None, None)
+    assert rc == -1 and b"temperature" in lib.rlk_last_error()
+
+
+def test_missing_library_fails_loudly(native, monkeypatch, tmp_path):
+    monkeypatch.setattr(native, "_lib", None)
+    monkeypatch.setattr(native, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(native.NativeLibraryError, match="no CPU or PyTorch fallback"):
+        native.load()
+    assert native.available() is False
