@@ -18,6 +18,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace rlk {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -148,6 +150,37 @@ struct TileIO {
         }
     }
 
+    // Single-pass forms used by the software-pipelined main loop.  CHECKED: a chunk at k >= K is
+    // fetched from a clamped (valid) address and replaced by zeros when it is stored to LDS.
+    __device__ inline bool live(int kt, int K, int p) const
+    {
+        const int t = threadIdx.x;
+        const int k = kt * BK + (KMAJOR ? p * G::kLinesPerPass + t / G::kChunksPerLine
+                                        : (t % G::kChunksPerLine) * 8);
+        return k < K;
+    }
+
+    template <bool CHECKED>
+    __device__ inline void load_one(int kt, int K, u32x4_t (&reg)[G::kPasses], int p) const
+    {
+        const uint32_t adv = static_cast<uint32_t>(kt) * step;
+        uint32_t o = off[p] + adv;
+        if (CHECKED) o = live(kt, K, p) ? o : off[p];
+        reg[p] = *reinterpret_cast<const u32x4_t*>(base + o);
+    }
+
+    template <bool CHECKED>
+    __device__ inline void store_one(char* lds, const u32x4_t (&reg)[G::kPasses], int p, int kt,
+                                     int K) const
+    {
+        const int t = threadIdx.x;
+        const int chunk = t % G::kChunksPerLine;
+        const int line = p * G::kLinesPerPass + t / G::kChunksPerLine;
+        u32x4_t v = reg[p];
+        if (CHECKED) v = live(kt, K, p) ? v : u32x4_t{0u, 0u, 0u, 0u};
+        *reinterpret_cast<u32x4_t*>(lds + line * G::kPitch + chunk * 16) = v;
+    }
+
     __device__ static inline void store(char* lds, const u32x4_t (&reg)[G::kPasses])
     {
         const int t = threadIdx.x;
@@ -185,72 +218,146 @@ struct TileIO {
     }
 };
 
+// Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
+template <int B, int E, class F>
+__device__ inline void static_for(F&& f)
+{
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
 // Workgroup tile contraction.  acc[i][j] (+)= A rows x B rows over k in [0, K).
 // smem must hold 2 * (A tile + B tile) bytes.  All 256 threads must call it (it barriers).
+//
+// The K loop is software pipelined by hand and the issue order is pinned with scheduling
+// barriers: every MFMA is followed by at most a couple of memory instructions, so LDS
+// fragment reads (for the next 16-wide k slice), LDS stores (next K step) and global loads
+// (the K step after that) all travel under the shadow of the matrix pipe.
+//   K step kt:  slice 0   : MFMAs | fragment reads for slice 1 | LDS stores of K step kt+1
+//               slice 1   : MFMAs | fragment reads for slice 2 | global loads of K step kt+2
+//               ...
+//               barrier
+//               last slice: MFMAs | fragment reads for slice 0 of K step kt+1
 template <class T, bool A_KMAJOR, bool B_KMAJOR, int TM, int TN, int BK>
 struct TileGemm {
     static constexpr int BM = 2 * TM * 32;
     static constexpr int BN = 2 * TN * 32;
+    static constexpr int KK = BK / 16;
+    static_assert(KK >= 2 && KK % 2 == 0, "BK must be 32 or 64");
     using IOA = TileIO<A_KMAJOR, BM, BK>;
     using IOB = TileIO<B_KMAJOR, BN, BK>;
+    static constexpr int PA = IOA::G::kPasses;
+    static constexpr int PB = IOB::G::kPasses;
     static constexpr int kStageBytes = IOA::G::kBytes + IOB::G::kBytes;
     static constexpr int kSmemBytes = 2 * kStageBytes;
+
+    // One 16-wide k slice of K step kt: TM*TN MFMAs from fragment set (KKI & 1), with this
+    // slice's share of memory instructions spread between them.  The loop body is identical for
+    // every K step (the K steps past the end re-fetch the last one into buffers nobody reads),
+    // which keeps the accumulator in one fixed set of registers.
+    template <int KKI, bool CHECKED>
+    __device__ static inline void slice(const IOA& la, const IOB& lb, u32x4_t (&ra)[PA],
+                                        u32x4_t (&rb)[PB], u32x4_t (&fa)[2][TM],
+                                        u32x4_t (&fb)[2][TN], int wm, int wn, int kstore, int kload,
+                                        int K,
+                                        const char* cur, char* nxt, f32x16_t (&acc)[TM][TN])
+    {
+        constexpr bool last = KKI == KK - 1;
+        constexpr int setc = KKI & 1, setn = setc ^ 1;
+        constexpr int NR = TM + TN;
+        constexpr int NW = KKI == 0 ? PA + PB : 0;
+        constexpr int NL = KKI == 1 ? PA + PB : 0;
+        constexpr int NOPS = NR + NW + NL;
+        constexpr int NM = TM * TN;
+        const char* rsrc = last ? nxt : cur;
+        constexpr int kkn = last ? 0 : KKI + 1;
+        static_for<0, NM>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            constexpr int i = q / TN, j = q % TN;
+            acc[i][j] = T::mfma(fa[setc][i], fb[setc][j], acc[i][j]);
+            static_for<q * NOPS / NM, (q + 1) * NOPS / NM>([&](auto oc) {
+                constexpr int o = decltype(oc)::value;
+                if constexpr (o < NR) {
+                    if constexpr (o < TM)
+                        fa[setn][o] = IOA::frag(rsrc, wm * (TM * 32) + o * 32, kkn);
+                    else
+                        fb[setn][o - TM] =
+                            IOB::frag(rsrc + IOA::G::kBytes, wn * (TN * 32) + (o - TM) * 32, kkn);
+                } else if constexpr (o < NR + NW) {
+                    constexpr int w = o - NR;
+                    if constexpr (w < PA)
+                        la.template store_one<CHECKED>(nxt, ra, w, kstore, K);
+                    else
+                        lb.template store_one<CHECKED>(nxt + IOA::G::kBytes, rb, w - PA, kstore, K);
+                } else {
+                    constexpr int g = o - NR - NW;
+                    if constexpr (g < PA)
+                        la.template load_one<CHECKED>(kload, K, ra, g);
+                    else
+                        lb.template load_one<CHECKED>(kload, K, rb, g - PA);
+                }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    }
+
+    template <bool CHECKED>
+    __device__ static inline void run_impl(const Operand& A, const Operand& B, int K,
+                                           f32x16_t (&acc)[TM][TN], char* smem)
+    {
+        IOA la;
+        IOB lb;
+        u32x4_t ra[PA];
+        u32x4_t rb[PB];
+        u32x4_t fa[2][TM];
+        u32x4_t fb[2][TN];
+        const int wave = threadIdx.x >> 6;
+        const int wm = wave >> 1;
+        const int wn = wave & 1;
+        la.init(A, K);
+        lb.init(B, K);
+        const int nk = (K + BK - 1) / BK;
+
+        la.template load<CHECKED>(0, K, ra);
+        lb.template load<CHECKED>(0, K, rb);
+        IOA::store(smem, ra);
+        IOB::store(smem + IOA::G::kBytes, rb);
+        {
+            const int k1 = nk > 1 ? 1 : 0;
+            la.template load<CHECKED>(k1, K, ra);
+            lb.template load<CHECKED>(k1, K, rb);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[0][i] = IOA::frag(smem, wm * (TM * 32) + i * 32, 0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            fb[0][j] = IOB::frag(smem + IOA::G::kBytes, wn * (TN * 32) + j * 32, 0);
+
+        for (int kt = 0; kt < nk; ++kt) {
+            const char* cur = smem + (kt & 1) * kStageBytes;
+            char* nxt = smem + ((kt + 1) & 1) * kStageBytes;
+            const int kstore = kt + 1 < nk ? kt + 1 : nk - 1;  // K step held in ra/rb
+            const int kload = kt + 2 < nk ? kt + 2 : nk - 1;
+            static_for<0, KK - 1>([&](auto kc) {
+                slice<decltype(kc)::value, CHECKED>(la, lb, ra, rb, fa, fb, wm, wn, kstore, kload, K,
+                                                    cur, nxt, acc);
+            });
+            __syncthreads();
+            slice<KK - 1, CHECKED>(la, lb, ra, rb, fa, fb, wm, wn, kstore, kload, K, cur, nxt, acc);
+        }
+        __syncthreads();  // LDS may be reused by the caller
+    }
 
     __device__ static inline void run(const Operand& A, const Operand& B, int K,
                                       f32x16_t (&acc)[TM][TN], char* smem)
     {
-        const int wave = threadIdx.x >> 6;
-        const int wm = wave >> 1;
-        const int wn = wave & 1;
-        u32x4_t ra[IOA::G::kPasses];
-        u32x4_t rb[IOB::G::kPasses];
-
-        IOA la;
-        IOB lb;
-        la.init(A, K);
-        lb.init(B, K);
-        const int nk = (K + BK - 1) / BK;
-        const int nfull = K / BK;  // K steps that need no bounds check
-        la.template load<true>(0, K, ra);
-        lb.template load<true>(0, K, rb);
-        IOA::store(smem, ra);
-        IOB::store(smem + IOA::G::kBytes, rb);
-        __syncthreads();
-
-        for (int kt = 0; kt < nk; ++kt) {
-            char* cur = smem + (kt & 1) * kStageBytes;
-            char* nxt = smem + ((kt + 1) & 1) * kStageBytes;
-            const bool more = kt + 1 < nk;
-            if (more) {
-                if (kt + 1 < nfull) {
-                    la.template load<false>(kt + 1, K, ra);
-                    lb.template load<false>(kt + 1, K, rb);
-                } else {
-                    la.template load<true>(kt + 1, K, ra);
-                    lb.template load<true>(kt + 1, K, rb);
-                }
-            }
-            const char* sa = cur;
-            const char* sb = cur + IOA::G::kBytes;
-#pragma unroll
-            for (int kk = 0; kk < BK / 16; ++kk) {
-                u32x4_t fa[TM];
-                u32x4_t fb[TN];
-#pragma unroll
-                for (int i = 0; i < TM; ++i) fa[i] = IOA::frag(sa, wm * (TM * 32) + i * 32, kk);
-#pragma unroll
-                for (int j = 0; j < TN; ++j) fb[j] = IOB::frag(sb, wn * (TN * 32) + j * 32, kk);
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) acc[i][j] = T::mfma(fa[i], fb[j], acc[i][j]);
-            }
-            if (more) {
-                IOA::store(nxt, ra);
-                IOB::store(nxt + IOA::G::kBytes, rb);
-            }
-            __syncthreads();
-        }
+        if (K % BK == 0)
+            run_impl<false>(A, B, K, acc, smem);
+        else
+            run_impl<true>(A, B, K, acc, smem);
     }
 };
 

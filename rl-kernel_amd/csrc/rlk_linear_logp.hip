@@ -355,34 +355,44 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     Gemm::run(A, B, a.v_valid, acc, smem);
 
+    // Epilogue: all reads of the running fp32 partial are issued before the first use (clamped
+    // addresses instead of branches), then added and stored under a predicate.
     const float oscale = a.scales[1];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int tl = tok0 + wn * 128 + j * 32 + (lane & 31);
-        if (tl >= a.tok_valid) continue;
+        const bool tok_ok = tl < a.tok_valid;
+        const int64_t trow = static_cast<int64_t>(tok_ok ? tl : a.tok_valid - 1) * a.H;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i) {
+            f32x4_t old[4];
+            int hcol[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int h = h0 + wm * 128 + i * 32 + 8 * q + 4 * (lane >> 5);
-                if (h >= a.H) continue;  // H % 8 == 0: the quad is all-in or all-out
+                hcol[q] = h;
+                old[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                if (!a.first)  // uniform
+                    old[q] = *reinterpret_cast<const f32x4_t*>(a.acc + trow + (h < a.H ? h : 0));
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
                 f32x4_t v{acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
                           acc[i][j][q * 4 + 3]};
-                float* ap = a.acc + static_cast<int64_t>(tl) * a.H + h;
-                if (!a.first) {
-                    const f32x4_t old = *reinterpret_cast<const f32x4_t*>(ap);
-                    v += old;
-                }
-                if (a.last) {
-                    u32x2_t pk{static_cast<uint32_t>(T::from_float(v.x * oscale)) |
-                                   (static_cast<uint32_t>(T::from_float(v.y * oscale)) << 16),
-                               static_cast<uint32_t>(T::from_float(v.z * oscale)) |
-                                   (static_cast<uint32_t>(T::from_float(v.w * oscale)) << 16)};
-                    *reinterpret_cast<u32x2_t*>(a.out + static_cast<int64_t>(tl) * a.H + h) = pk;
-                } else {
-                    *reinterpret_cast<f32x4_t*>(ap) = v;
+                v += old[q];
+                if (tok_ok && hcol[q] < a.H) {  // H % 8 == 0: a quad is all-in or all-out
+                    if (a.last) {
+                        u32x2_t pk{static_cast<uint32_t>(T::from_float(v.x * oscale)) |
+                                       (static_cast<uint32_t>(T::from_float(v.y * oscale)) << 16),
+                                   static_cast<uint32_t>(T::from_float(v.z * oscale)) |
+                                       (static_cast<uint32_t>(T::from_float(v.w * oscale)) << 16)};
+                        *reinterpret_cast<u32x2_t*>(a.out + trow + hcol[q]) = pk;
+                    } else {
+                        *reinterpret_cast<f32x4_t*>(a.acc + trow + hcol[q]) = v;
+                    }
                 }
             }
+        }
     }
 }
 
@@ -427,22 +437,31 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     Gemm::run(A, B, a.tok_valid, acc, smem);
 
+    // Epilogue: read-modify-write of the fp32 dW tile; the 16 reads of one MFMA tile are issued
+    // together (clamped addresses), then added and stored under a predicate.
     const float oscale = a.scales[1];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int h = h0 + wn * 128 + j * 32 + (lane & 31);
-        if (h >= a.H) continue;
+        const bool h_ok = h < a.H;
+        const int hc = h_ok ? h : 0;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i) {
+            float old[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int v = v0 + wm * 128 + i * 32 + acc_row(r, lane);
-                if (v >= a.v_valid) continue;
-                float* p = a.dw + static_cast<int64_t>(v) * a.H + h;
-                float val = acc[i][j][r] * oscale;
-                if (a.accumulate) val += *p;
-                *p = val;
+                old[r] = 0.f;
+                if (a.accumulate)  // uniform
+                    old[r] = a.dw[static_cast<int64_t>(v < a.v_valid ? v : a.v_valid - 1) * a.H + hc];
             }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int v = v0 + wm * 128 + i * 32 + acc_row(r, lane);
+                if (h_ok && v < a.v_valid)
+                    a.dw[static_cast<int64_t>(v) * a.H + h] = fmaf(acc[i][j][r], oscale, old[r]);
+            }
+        }
     }
 }
 
