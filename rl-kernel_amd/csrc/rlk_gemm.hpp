@@ -34,6 +34,12 @@ typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 
 #define RLK_LDS __attribute__((address_space(3)))
 
+// Development switch for timing experiments (wrong results when non-zero): bit 0 drops the
+// global loads of the main loop, bit 1 the LDS stores, bit 2 the fragment reads, bit 3 the barrier.
+#ifndef RLK_ABLATE
+#define RLK_ABLATE 0
+#endif
+
 constexpr int kThreads = 256;
 
 struct Bf16 {
@@ -235,11 +241,11 @@ __device__ inline void static_for(F&& f)
 // barriers: every MFMA is followed by at most a couple of memory instructions, so LDS
 // fragment reads (for the next 16-wide k slice), LDS stores (next K step) and global loads
 // (the K step after that) all travel under the shadow of the matrix pipe.
-//   K step kt:  slice 0   : MFMAs | fragment reads for slice 1 | LDS stores of K step kt+1
-//               slice 1   : MFMAs | fragment reads for slice 2 | global loads of K step kt+2
-//               ...
+//   K step kt:  slices 0..KK-2: MFMAs | fragment reads for the next slice
+//                               | every few MFMAs: one LDS store of K step kt+1, then the global
+//                                 load of K step kt+2 into the registers that store just freed
 //               barrier
-//               last slice: MFMAs | fragment reads for slice 0 of K step kt+1
+//               last slice    : MFMAs | fragment reads for slice 0 of K step kt+1
 template <class T, bool A_KMAJOR, bool B_KMAJOR, int TM, int TN, int BK>
 struct TileGemm {
     static constexpr int BM = 2 * TM * 32;
@@ -267,38 +273,45 @@ struct TileGemm {
         constexpr bool last = KKI == KK - 1;
         constexpr int setc = KKI & 1, setn = setc ^ 1;
         constexpr int NR = TM + TN;
-        constexpr int NW = KKI == 0 ? PA + PB : 0;
-        constexpr int NL = KKI == 1 ? PA + PB : 0;
-        constexpr int NOPS = NR + NW + NL;
         constexpr int NM = TM * TN;
+        constexpr int NW = PA + PB;                  // LDS stores == global loads per K step
+        constexpr int SP = (NM * (KK - 1)) / NW;     // MFMA slots between consecutive stores
+        static_assert(SP >= 2, "not enough MFMA slots before the barrier");
         const char* rsrc = last ? nxt : cur;
         constexpr int kkn = last ? 0 : KKI + 1;
         static_for<0, NM>([&](auto qc) {
             constexpr int q = decltype(qc)::value;
             constexpr int i = q / TN, j = q % TN;
+            constexpr int slot = KKI * NM + q;       // MFMA index inside the K step
             acc[i][j] = T::mfma(fa[setc][i], fb[setc][j], acc[i][j]);
-            static_for<q * NOPS / NM, (q + 1) * NOPS / NM>([&](auto oc) {
+            // fragment reads for the next slice, spread evenly over this slice
+            static_for<q * NR / NM, (q + 1) * NR / NM>([&](auto oc) {
                 constexpr int o = decltype(oc)::value;
-                if constexpr (o < NR) {
-                    if constexpr (o < TM)
-                        fa[setn][o] = IOA::frag(rsrc, wm * (TM * 32) + o * 32, kkn);
-                    else
-                        fb[setn][o - TM] =
-                            IOB::frag(rsrc + IOA::G::kBytes, wn * (TN * 32) + (o - TM) * 32, kkn);
-                } else if constexpr (o < NR + NW) {
-                    constexpr int w = o - NR;
-                    if constexpr (w < PA)
-                        la.template store_one<CHECKED>(nxt, ra, w, kstore, K);
-                    else
-                        lb.template store_one<CHECKED>(nxt + IOA::G::kBytes, rb, w - PA, kstore, K);
-                } else {
-                    constexpr int g = o - NR - NW;
-                    if constexpr (g < PA)
-                        la.template load_one<CHECKED>(kload, K, ra, g);
-                    else
-                        lb.template load_one<CHECKED>(kload, K, rb, g - PA);
-                }
+                if constexpr ((RLK_ABLATE & 4) != 0) {
+                } else if constexpr (o < TM)
+                    fa[setn][o] = IOA::frag(rsrc, wm * (TM * 32) + o * 32, kkn);
+                else
+                    fb[setn][o - TM] =
+                        IOB::frag(rsrc + IOA::G::kBytes, wn * (TN * 32) + (o - TM) * 32, kkn);
             });
+            // pass w: LDS store at slot w*SP, the global load that refills the same registers
+            // right after it, so loads are spaced evenly and get a full K step of latency
+            if constexpr (slot % SP == 0 && slot / SP < NW) {
+                constexpr int w = slot / SP;
+                if constexpr ((RLK_ABLATE & 2) != 0) {
+                } else if constexpr (w < PA)
+                    la.template store_one<CHECKED>(nxt, ra, w, kstore, K);
+                else
+                    lb.template store_one<CHECKED>(nxt + IOA::G::kBytes, rb, w - PA, kstore, K);
+            }
+            if constexpr (slot % SP == 1 && slot / SP < NW) {
+                constexpr int g = slot / SP;
+                if constexpr ((RLK_ABLATE & 1) != 0) {
+                } else if constexpr (g < PA)
+                    la.template load_one<CHECKED>(kload, K, ra, g);
+                else
+                    lb.template load_one<CHECKED>(kload, K, rb, g - PA);
+            }
             __builtin_amdgcn_sched_barrier(0);
         });
     }
@@ -345,8 +358,14 @@ struct TileGemm {
                 slice<decltype(kc)::value, CHECKED>(la, lb, ra, rb, fa, fb, wm, wn, kstore, kload, K,
                                                     cur, nxt, acc);
             });
-            __syncthreads();
+            if constexpr ((RLK_ABLATE & 8) == 0) __syncthreads();
             slice<KK - 1, CHECKED>(la, lb, ra, rb, fa, fb, wm, wn, kstore, kload, K, cur, nxt, acc);
+        }
+        if constexpr ((RLK_ABLATE & 16) != 0) {  // keep the (unused) global loads alive
+#pragma unroll
+            for (int p = 0; p < PA; ++p) asm volatile("" ::"v"(ra[p]));
+#pragma unroll
+            for (int p = 0; p < PB; ++p) asm volatile("" ::"v"(rb[p]));
         }
         __syncthreads();  // LDS may be reused by the caller
     }
