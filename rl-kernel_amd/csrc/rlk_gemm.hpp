@@ -1,8 +1,8 @@
 // MFMA tile GEMM mainloop for gfx950 (CDNA4), shared by the four contraction kernels of the
 // fused linear-logprob path (forward logits tile, dZ recompute, dH, dW).
 //
-// One workgroup = 256 threads = 4 wavefronts arranged 2 (M) x 2 (N).  The workgroup computes a
-// (2*TM*32) x (2*TN*32) tile D = A * B^T-like contraction over K with v_mfma_f32_32x32x16
+// One workgroup = kWM x kWN wavefronts (2 x 4 by default).  The workgroup computes a
+// 256 x 256 tile D = A * B^T-like contraction over K with v_mfma_f32_32x32x16
 // (bf16 or f16 inputs, fp32 accumulate); each wavefront owns TM x TN MFMA tiles of 32x32.
 //
 // Operands are described by (base pointer at the tile origin, leading dimension, valid rows):
@@ -40,7 +40,20 @@ typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 #define RLK_ABLATE 0
 #endif
 
-constexpr int kThreads = 256;
+// Workgroup shape: kWM x kWN wavefronts tile the 256 x 256 block; each wavefront owns
+// kTM x kTN MFMA tiles of 32 x 32.
+#ifndef RLK_WM
+#define RLK_WM 2
+#endif
+#ifndef RLK_WN
+#define RLK_WN 4
+#endif
+constexpr int kWM = RLK_WM;
+constexpr int kWN = RLK_WN;
+constexpr int kThreads = 64 * kWM * kWN;
+constexpr int kTM = 256 / (32 * kWM);
+constexpr int kTN = 256 / (32 * kWN);
+static_assert(kTM * kWM * 32 == 256 && kTN * kWN * 32 == 256, "wave grid must tile 256 x 256");
 
 struct Bf16 {
     static constexpr int kId = 0;
@@ -246,10 +259,12 @@ __device__ inline void static_for(F&& f)
 //                                 load of K step kt+2 into the registers that store just freed
 //               barrier
 //               last slice    : MFMAs | fragment reads for slice 0 of K step kt+1
-template <class T, bool A_KMAJOR, bool B_KMAJOR, int TM, int TN, int BK>
+template <class T, bool A_KMAJOR, bool B_KMAJOR, int BK>
 struct TileGemm {
-    static constexpr int BM = 2 * TM * 32;
-    static constexpr int BN = 2 * TN * 32;
+    static constexpr int TM = kTM;
+    static constexpr int TN = kTN;
+    static constexpr int BM = kWM * TM * 32;
+    static constexpr int BN = kWN * TN * 32;
     static constexpr int KK = BK / 16;
     static_assert(KK >= 2 && KK % 2 == 0, "BK must be 32 or 64");
     using IOA = TileIO<A_KMAJOR, BM, BK>;
@@ -327,8 +342,8 @@ struct TileGemm {
         u32x4_t fa[2][TM];
         u32x4_t fb[2][TN];
         const int wave = threadIdx.x >> 6;
-        const int wm = wave >> 1;
-        const int wn = wave & 1;
+        const int wm = wave / kWN;
+        const int wn = wave % kWN;
         la.init(A, K);
         lb.init(B, K);
         const int nk = (K + BK - 1) / BK;

@@ -37,14 +37,14 @@ struct FwdArgs {
     float scale2;    // log2(e) / temperature
 };
 
-// Online-softmax update of one wavefront slab (128 vocab rows x 128 tokens) held in `acc`.
+// Online-softmax update of one wavefront slab (kTM*32 vocab rows x kTN*32 tokens) held in `acc`.
 // GENERAL = false: no bias and no masked vocab rows (every tile full), the common case.
 // The target logit is picked up in the same pass that feeds the sum, so the captured value is
 // the very fp32 number that entered the softmax.
 template <bool GENERAL>
-__device__ inline void fwd_epilogue(const f32x16_t (&acc)[4][4], const FwdArgs& a, int vw, int lane,
-                                    const int (&tgt)[4], float (&m)[4], float (&s)[4],
-                                    float (&zt)[4])
+__device__ inline void fwd_epilogue(const f32x16_t (&acc)[kTM][kTN], const FwdArgs& a, int vw,
+                                    int lane, const int (&tgt)[kTN], float (&m)[kTN],
+                                    float (&s)[kTN], float (&zt)[kTN])
 {
     auto logit = [&](int i, int j, int r) -> float {
         float z = acc[i][j][r];
@@ -56,10 +56,10 @@ __device__ inline void fwd_epilogue(const f32x16_t (&acc)[4][4], const FwdArgs& 
         return z;
     };
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kTN; ++j) {
         float tmax = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < kTM; ++i)
 #pragma unroll
             for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, logit(i, j, r));
         __builtin_amdgcn_sched_barrier(0);
@@ -69,12 +69,12 @@ __device__ inline void fwd_epilogue(const f32x16_t (&acc)[4][4], const FwdArgs& 
         // register index (i*16 + r) of the target row in this lane, or -1
         const int tl = tgt[j] - vw;
         const int x = tl & 31;
-        const int etgt = (static_cast<unsigned>(tl) < 128u && ((x >> 2) & 1) == (lane >> 5))
+        const int etgt = (static_cast<unsigned>(tl) < static_cast<unsigned>(kTM * 32) && ((x >> 2) & 1) == (lane >> 5))
                              ? ((tl >> 5) * 16 + (x >> 3) * 4 + (x & 3))
                              : -1;
         float sum = 0.f, zraw = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < kTM; ++i)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float z = logit(i, j, r);
@@ -94,8 +94,8 @@ __device__ inline void fwd_epilogue(const f32x16_t (&acc)[4][4], const FwdArgs& 
 template <class T, int BK, bool GENERAL>
 __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
 {
-    constexpr int TM = 4, TN = 4;
-    using Gemm = TileGemm<T, false, false, TM, TN, BK>;
+    constexpr int TM = kTM, TN = kTN;
+    using Gemm = TileGemm<T, false, false, BK>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     int tb, sp;
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / kWN, wn = wave % kWN;
     const int tok0 = tb * 256;
     const int tok_valid = min(256, a.N - tok0);
 
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
         m[j] = -INFINITY;
         s[j] = 0.f;
         zt[j] = 0.f;
-        const int t = wn * 128 + j * 32 + (lane & 31);
+        const int t = wn * (TN * 32) + j * 32 + (lane & 31);
         int64_t g = a.targets[tok0 + (t < tok_valid ? t : tok_valid - 1)] - a.vocab_start;
         tgt[j] = (g >= 0 && g < a.V) ? static_cast<int>(g) : -1;
     }
@@ -135,12 +135,12 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
         Gemm::run(A, B, a.H, acc, smem);
-        fwd_epilogue<GENERAL>(acc, a, v0 + wm * 128, lane, tgt, m, s, zt);
+        fwd_epilogue<GENERAL>(acc, a, v0 + wm * (TM * 32), lane, tgt, m, s, zt);
     }
 
     // Merge the two half-wave row groups (same token, different vocab rows), then the two
     // wavefronts along M through LDS, in a fixed order.
-    float* red = reinterpret_cast<float*>(smem);  // [2 (wm)][256 tokens][3]
+    float* red = reinterpret_cast<float*>(smem);  // [kWM][256 tokens][3]
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const float m2 = __shfl_xor(m[j], 32);
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
         const float ss = lo_s * __builtin_amdgcn_exp2f(lo_m - mref) +
                          hi_s * __builtin_amdgcn_exp2f(hi_m - mref);
         if (lane < 32) {
-            float* dst = red + ((wm * 256) + wn * 128 + j * 32 + lane) * 3;
+            float* dst = red + ((wm * 256) + wn * (TN * 32) + j * 32 + lane) * 3;
             dst[0] = mm;
             dst[1] = ss;
             dst[2] = zt[j] + z2;
@@ -162,16 +162,21 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
     __syncthreads();
     const int t = threadIdx.x;
     if (t < tok_valid) {
-        const float* p0 = red + t * 3;
-        const float* p1 = red + (256 + t) * 3;
-        const float mm = fmaxf(p0[0], p1[0]);
+        float mm = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWM; ++w) mm = fmaxf(mm, red[(w * 256 + t) * 3]);
         const float mref = mm == -INFINITY ? 0.f : mm;
-        const float ss = p0[1] * __builtin_amdgcn_exp2f(p0[0] - mref) +
-                         p1[1] * __builtin_amdgcn_exp2f(p1[0] - mref);
+        float ss = 0.f, zz = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWM; ++w) {
+            const float* pw = red + (w * 256 + t) * 3;
+            ss += pw[1] * __builtin_amdgcn_exp2f(pw[0] - mref);
+            zz += pw[2];
+        }
         const int64_t o = static_cast<int64_t>(a.split_lo + sp) * a.N + tok0 + t;
         a.part_m[o] = mm;
         a.part_s[o] = ss;
-        a.part_z[o] = p0[2] + p1[2];
+        a.part_z[o] = zz;
     }
 }
 
@@ -244,15 +249,15 @@ struct DzArgs {
 template <class T, int BK, bool GENERAL>
 __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
 {
-    constexpr int TM = 4, TN = 4;
-    using Gemm = TileGemm<T, false, false, TM, TN, BK>;
+    constexpr int TM = kTM, TN = kTN;
+    using Gemm = TileGemm<T, false, false, BK>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     int vt, tt;
     xcd_tile(blockIdx.x, a.tok_tiles * a.v_tiles, a.v_tiles, a.tok_tiles, 8, vt, tt);
     vt += a.v_tile_lo;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / kWN, wn = wave % kWN;
     const int tok0 = tt * 256, v0 = vt * 256;
     const int tok_rows = min(256, a.tok_valid - tok0);
     const int v_rows = min(256, a.v_valid - v0);
@@ -269,10 +274,10 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
     Gemm::run(A, B, a.H, acc, smem);
 
     const float gscale = a.scales[0];
-    const int vw = v0 + wm * 128;
+    const int vw = v0 + wm * (TM * 32);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int tl = wn * 128 + j * 32 + (lane & 31);
+        const int tl = wn * (TN * 32) + j * 32 + (lane & 31);
         const int tc = tok0 + (tl < tok_rows ? tl : tok_rows - 1);
         const int64_t tg = a.targets[tc];
         const bool live = tl < tok_rows && !(a.use_ignore && tg == a.ignore_index);
@@ -280,7 +285,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
         const float nlse2 = -a.lse[tc] * kLog2e;
         // register index (i*16 + r) of the target row in this lane, or -1
         const int64_t trel = tg - a.v_global0 - vw;
-        const int tr = (trel >= 0 && trel < 128) ? static_cast<int>(trel) : -1;
+        const int tr = (trel >= 0 && trel < TM * 32) ? static_cast<int>(trel) : -1;
         const int x = tr & 31;
         const int etgt = (tr >= 0 && ((x >> 2) & 1) == (lane >> 5))
                              ? ((tr >> 5) * 16 + (x >> 3) * 4 + (x & 3))
@@ -334,14 +339,14 @@ struct DhArgs {
 template <class T, int BK>
 __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
 {
-    constexpr int TM = 4, TN = 4;
-    using Gemm = TileGemm<T, true, false, TM, TN, BK>;
+    constexpr int TM = kTM, TN = kTN;
+    using Gemm = TileGemm<T, true, false, BK>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     int tt, ht;
     xcd_tile(blockIdx.x, a.tok_tiles * a.h_tiles, a.tok_tiles, a.h_tiles, 8, tt, ht);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / kWN, wn = wave % kWN;
     const int tok0 = tt * 256, h0 = ht * 256;
 
     Operand A{a.weight + h0, a.H, min(256, a.H - h0)};
@@ -360,7 +365,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
     const float oscale = a.scales[1];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int tl = tok0 + wn * 128 + j * 32 + (lane & 31);
+        const int tl = tok0 + wn * (TN * 32) + j * 32 + (lane & 31);
         const bool tok_ok = tl < a.tok_valid;
         const int64_t trow = static_cast<int64_t>(tok_ok ? tl : a.tok_valid - 1) * a.H;
 #pragma unroll
@@ -369,7 +374,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
             int hcol[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int h = h0 + wm * 128 + i * 32 + 8 * q + 4 * (lane >> 5);
+                const int h = h0 + wm * (TM * 32) + i * 32 + 8 * q + 4 * (lane >> 5);
                 hcol[q] = h;
                 old[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
                 if (!a.first)  // uniform
@@ -416,14 +421,14 @@ struct DwArgs {
 template <class T, int BK>
 __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
 {
-    constexpr int TM = 4, TN = 4;
-    using Gemm = TileGemm<T, true, true, TM, TN, BK>;
+    constexpr int TM = kTM, TN = kTN;
+    using Gemm = TileGemm<T, true, true, BK>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     int vt, ht;
     xcd_tile(blockIdx.x, a.v_tiles * a.h_tiles, a.v_tiles, a.h_tiles, 8, vt, ht);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / kWN, wn = wave % kWN;
     const int v0 = vt * 256, h0 = ht * 256;
 
     Operand A{a.dz + v0, a.ldz, 256};
@@ -442,7 +447,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
     const float oscale = a.scales[1];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int h = h0 + wn * 128 + j * 32 + (lane & 31);
+        const int h = h0 + wn * (TN * 32) + j * 32 + (lane & 31);
         const bool h_ok = h < a.H;
         const int hc = h_ok ? h : 0;
 #pragma unroll
@@ -450,14 +455,14 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
             float old[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int v = v0 + wm * 128 + i * 32 + acc_row(r, lane);
+                const int v = v0 + wm * (TM * 32) + i * 32 + acc_row(r, lane);
                 old[r] = 0.f;
                 if (a.accumulate)  // uniform
                     old[r] = a.dw[static_cast<int64_t>(v < a.v_valid ? v : a.v_valid - 1) * a.H + hc];
             }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int v = v0 + wm * 128 + i * 32 + acc_row(r, lane);
+                const int v = v0 + wm * (TM * 32) + i * 32 + acc_row(r, lane);
                 if (h_ok && v < a.v_valid)
                     a.dw[static_cast<int64_t>(v) * a.H + h] = fmaf(acc[i][j][r], oscale, old[r]);
             }
@@ -689,7 +694,7 @@ int rlk_linear_logp_fwd(const void* hidden, const void* weight, const float* bia
     a.part_z = a.part_s + static_cast<size_t>(plan.total_splits) * N;
     a.scale2 = kLog2e / temperature;
 
-    using G = TileGemm<Bf16, false, false, 4, 4, kBK>;  // same LDS footprint for f16
+    using G = TileGemm<Bf16, false, false, kBK>;  // same LDS footprint for f16
     if (plan.n_fast > 0) {
         a.n_split = plan.n_fast;
         a.split_lo = 0;
@@ -793,9 +798,9 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                        static_cast<int>(N), 1.f / temperature, dtype, scales);
     if (int rc = check_launch("scales kernel launch failed")) return rc;
 
-    using GZb = TileGemm<Bf16, false, false, 4, 4, kBK>;
-    using GHb = TileGemm<Bf16, true, false, 4, 4, kBK>;
-    using GWb = TileGemm<Bf16, true, true, 4, 4, kBK>;
+    using GZb = TileGemm<Bf16, false, false, kBK>;
+    using GHb = TileGemm<Bf16, true, false, kBK>;
+    using GWb = TileGemm<Bf16, true, true, kBK>;
     if (dtype == RLK_DTYPE_BF16) {
         if (int rc = set_smem(linear_logp_dz_kernel<Bf16, kBK, false>, GZb::kSmemBytes)) return rc;
         if (int rc = set_smem(linear_logp_dz_kernel<Bf16, kBK, true>, GZb::kSmemBytes)) return rc;
