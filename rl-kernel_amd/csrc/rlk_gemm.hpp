@@ -299,15 +299,19 @@ struct TileGemm {
             constexpr int i = q / TN, j = q % TN;
             constexpr int slot = KKI * NM + q;       // MFMA index inside the K step
             acc[i][j] = T::mfma(fa[setc][i], fb[setc][j], acc[i][j]);
-            // fragment reads for the next slice, spread evenly over this slice
+            // fragment reads for the next slice, spread evenly over this slice and issued in the
+            // order the next slice's MFMAs (i-major) first need them: A0, B0..B(TN-1), A1..A(TM-1)
             static_for<q * NR / NM, (q + 1) * NR / NM>([&](auto oc) {
                 constexpr int o = decltype(oc)::value;
                 if constexpr ((RLK_ABLATE & 4) != 0) {
-                } else if constexpr (o < TM)
-                    fa[setn][o] = IOA::frag(rsrc, wm * (TM * 32) + o * 32, kkn);
-                else
-                    fb[setn][o - TM] =
-                        IOB::frag(rsrc + IOA::G::kBytes, wn * (TN * 32) + (o - TM) * 32, kkn);
+                } else if constexpr (o == 0 || o > TN) {
+                    constexpr int fi = o == 0 ? 0 : o - TN;
+                    fa[setn][fi] = IOA::frag(rsrc, wm * (TM * 32) + fi * 32, kkn);
+                } else {
+                    constexpr int fj = o - 1;
+                    fb[setn][fj] =
+                        IOB::frag(rsrc + IOA::G::kBytes, wn * (TN * 32) + fj * 32, kkn);
+                }
             });
             // pass w: LDS store at slot w*SP, the global load that refills the same registers
             // right after it, so loads are spaced evenly and get a full K step of latency
