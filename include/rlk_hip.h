@@ -68,8 +68,11 @@ const char* rlk_last_error(void);
  *            reference's ValueError (rl_engine/kernels/ops/cuda/loss/linear_logp.py:352-358).
  *            With strict_targets == 0 such a row yields logp = -lse (z_t = 0), which is what a
  *            vocab-parallel shard must return (csrc/cuda/fused_linear_logp_sm90.cu:256-280).
- *   H must be a multiple of 8 and the two matrices 16-byte aligned, else RLK_ERR_UNSUPPORTED /
- *   RLK_ERR_ARG.
+ *   dtype: RLK_DTYPE_BF16 / RLK_DTYPE_F16 with H % 8 == 0 and 16-byte aligned matrices run on the
+ *   MFMA tiles; RLK_DTYPE_F32, other H or misaligned matrices run on scalar-FMA kernels (same
+ *   math in fp32, H <= 12288) -- the counterpart of the reference's "unsupported dtype/shape falls
+ *   back to the portable op" (rl_engine/kernels/ops/cuda/loss/linear_logp.py:45-55,350-351),
+ *   except that here the portable op is HIP too.
  * ------------------------------------------------------------------------------------------ */
 int rlk_linear_logp_fwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                         size_t* bytes);
@@ -106,6 +109,65 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                         size_t workspace_bytes, size_t dz_budget_bytes, int64_t N, int32_t H,
                         int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
                         int64_t ignore_index, int32_t use_ignore, rlk_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------ *
+ * Selected-token log-prob from materialised logits (the `fused_logp` family).
+ *
+ * Stands in for the nine `_C.fused_logp*` symbols (csrc/ops.cpp:75-96, csrc/fused_logp_kernel.cu:
+ * 452-588; signatures in rl_engine/_C.pyi:5-43): one single-pass online-softmax scan serves the
+ * two-pass and the `online` variants alike (they compute the same value).
+ *   logits [n_rows, vocab] bf16/f16/f32, ids [n_rows] int64, out [n_rows] of out_dtype
+ *   (bf16/f16/f32/f64).  row_indices == NULL: every row is written (n_launch == n_rows).
+ *   row_indices != NULL: only the n_launch listed rows are written, the others are left
+ *   untouched; listed rows outside [0, n_rows) are skipped (csrc/fused_logp_kernel.cu:120-123).
+ *   An id outside [0, vocab) yields 0, not an error (same file :147-155).
+ *   lse_out (optional, f32 [n_rows]) receives logsumexp of each written row.
+ * ------------------------------------------------------------------------------------------ */
+int rlk_logp_from_logits(const void* logits, int32_t logits_dtype, const int64_t* ids, void* out,
+                         int32_t out_dtype, float* lse_out, const int64_t* row_indices,
+                         int64_t n_launch, int64_t n_rows, int64_t vocab, rlk_stream_t stream);
+
+/* Backward of the above w.r.t. the logits:
+ *   grad_logits[n][v] = coeff[n] * (onehot(ids[n])[v] - exp(logits[n][v] - lse[n]))
+ * in the logits dtype; rows whose id is outside [0, vocab) get zeros.  Stands in for the
+ * analytic backward of rl_engine/kernels/ops/triton/loss/ratio_kl.py:86-122 and for autograd
+ * through rl_engine/kernels/ops/pytorch/loss/logp.py:16-32. */
+int rlk_logp_from_logits_bwd(const void* logits, int32_t logits_dtype, const int64_t* ids,
+                             const float* lse, const float* coeff, void* grad_logits,
+                             int64_t n_rows, int64_t vocab, rlk_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------ *
+ * Log-prob-fed GRPO / PPO loss epilogue.
+ *
+ * Stands in for the composition compute_policy_ratio / compute_reference_kl / masked_mean
+ * (rl_engine/testing/reference_ops.py:50-106) as chained by
+ * rl_engine/executors/deepspeed_trainer.py:160-167 and
+ * rl_engine/kernels/ops/pytorch/loss/grpo_loss.py:96-125:
+ *   r = exp(cur - old) ; d = ref - cur ; M = max(sum(mask), 1e-8)
+ *   policy = sum(mask * -min(r A, clip(r, 1-eps, 1+eps) A)) / M
+ *   kl     = sum(mask * (e^d - d - 1)) / M               (0 when ref_logp == NULL)
+ *   out3   = { policy + beta * kl, policy, kl }
+ *   d_cur  = d out3[0] / d cur (optional; multiplied by *upstream when given)
+ *   d_kl   = d out3[2] / d cur (optional, needs d_cur; so d out3[1]/d cur = d_cur - beta * d_kl)
+ * advantages: per token [n_tokens] (adv_per_token != 0) or per sequence [n_tokens / seq_len].
+ * mask: uint8 [n_tokens] or NULL (all active).  ratio / kl_terms (optional) receive the per-token
+ * values with masked entries 0.  Sums use a fixed two-level tree.
+ * ------------------------------------------------------------------------------------------ */
+int rlk_grpo_loss_workspace_bytes(int64_t n_tokens, size_t* bytes);
+
+int rlk_grpo_loss_from_logp(const float* cur_logp, const float* old_logp, const float* ref_logp,
+                            const float* advantages, int32_t adv_per_token, const uint8_t* mask,
+                            int64_t n_tokens, int64_t seq_len, float clip_eps, float beta,
+                            float* out3, float* ratio, float* kl_terms, float* d_cur, float* d_kl,
+                            const float* upstream, void* workspace, size_t workspace_bytes,
+                            rlk_stream_t stream);
+
+/* Per-group reward normalisation (x - mean_g) / sqrt(max(E_g[x^2] - mean_g^2, eps^2)) over CSR
+ * group boundaries (int64 [num_groups + 1], device).  Stands in for
+ * NativeGRPOLossOp.group_advantages (rl_engine/kernels/ops/pytorch/loss/grpo_loss.py:53-84) and
+ * _group_norm_kernel (rl_engine/kernels/ops/triton/loss/grpo_loss.py:30-55). */
+int rlk_group_advantages(const float* rewards, const int64_t* group_bounds, int64_t num_groups,
+                         float eps, float* advantages, rlk_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------ *
  * Hardware-contract self test (no counterpart in the reference): checks that the gfx950

@@ -16,3 +16,18 @@
 
 // Records `msg` as the calling thread's last error and returns `code` (always negative).
 int rlk_fail(int code, const char* msg);
+
+// Scalar-FMA implementation of the same two entry points for what the MFMA tiles do not take:
+// fp32 inputs, hidden sizes that are not a multiple of 8, misaligned matrices (rlk_generic.hip).
+namespace rlk {
+int generic_fwd(const void* hidden, const void* weight, const float* bias, const int64_t* targets,
+                float* logp, float* lse, int64_t N, int32_t H, int64_t V, int64_t vocab_start,
+                int32_t dtype, float temperature, int64_t ignore_index, int32_t use_ignore,
+                int32_t strict_targets, int32_t* err_flag, hipStream_t stream);
+size_t generic_bwd_workspace(int64_t N, int32_t H, int64_t V);
+int generic_bwd(const float* grad_logp, const void* hidden, const void* weight, const float* bias,
+                const int64_t* targets, const float* lse, void* d_hidden, float* d_weight,
+                float* d_bias, void* workspace, int64_t N, int32_t H, int64_t V,
+                int64_t vocab_start, int32_t dtype, float temperature, int64_t ignore_index,
+                int32_t use_ignore, hipStream_t stream);
+}  // namespace rlk

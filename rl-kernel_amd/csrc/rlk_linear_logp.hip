@@ -636,16 +636,21 @@ int check_launch(const char* what)
     return 0;
 }
 
-int check_common(const void* hidden, const void* weight, int64_t N, int32_t H, int64_t V, int dtype)
+int check_common(int64_t N, int32_t H, int64_t V, int dtype)
 {
-    if (dtype != RLK_DTYPE_BF16 && dtype != RLK_DTYPE_F16)
-        return rlk_fail(RLK_ERR_UNSUPPORTED, "dtype must be RLK_DTYPE_BF16 or RLK_DTYPE_F16");
+    if (dtype != RLK_DTYPE_BF16 && dtype != RLK_DTYPE_F16 && dtype != RLK_DTYPE_F32)
+        return rlk_fail(RLK_ERR_UNSUPPORTED, "dtype must be RLK_DTYPE_BF16, RLK_DTYPE_F16 or RLK_DTYPE_F32");
     if (N <= 0 || H <= 0 || V <= 0) return rlk_fail(RLK_ERR_ARG, "N, H and V must be positive");
-    if (H % 8 != 0) return rlk_fail(RLK_ERR_UNSUPPORTED, "H must be a multiple of 8");
     if (N > 0x7fff0000LL || V > 0x7fff0000LL) return rlk_fail(RLK_ERR_ARG, "N or V too large");
-    if ((reinterpret_cast<uintptr_t>(hidden) & 15) || (reinterpret_cast<uintptr_t>(weight) & 15))
-        return rlk_fail(RLK_ERR_ARG, "hidden and weight must be 16-byte aligned");
     return 0;
+}
+
+// The MFMA tiles take 16-bit inputs whose rows start on 16-byte boundaries; everything else runs
+// on the scalar-FMA kernels.
+bool use_mfma(const void* hidden, const void* weight, int32_t H, int dtype)
+{
+    return (dtype == RLK_DTYPE_BF16 || dtype == RLK_DTYPE_F16) && H % 8 == 0 &&
+           (reinterpret_cast<uintptr_t>(hidden) & 15) == 0 && (reinterpret_cast<uintptr_t>(weight) & 15) == 0;
 }
 
 }  // namespace
@@ -671,9 +676,13 @@ int rlk_linear_logp_fwd(const void* hidden, const void* weight, const float* bia
                         int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
                         int32_t* err_flag, hipStream_t stream)
 {
-    if (int rc = check_common(hidden, weight, N, H, V, dtype)) return rc;
+    if (int rc = check_common(N, H, V, dtype)) return rc;
     if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
-    if (!targets || !logp || !lse || !err_flag) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (!hidden || !weight || !targets || !logp || !lse || !err_flag)
+        return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (!use_mfma(hidden, weight, H, dtype))
+        return generic_fwd(hidden, weight, bias, targets, logp, lse, N, H, V, vocab_start, dtype,
+                           temperature, ignore_index, use_ignore, strict_targets, err_flag, stream);
     size_t need = 0;
     rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &need);
     if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
@@ -762,7 +771,9 @@ int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t
     if (!bytes || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad workspace query");
     if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
     if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
-    *bytes = bwd_plan(N, H, V, dz_budget_bytes).total;
+    // large enough for either implementation (the choice also depends on pointer alignment)
+    const size_t a = bwd_plan(N, H, V, dz_budget_bytes).total, b = generic_bwd_workspace(N, H, V);
+    *bytes = a > b ? a : b;
     return 0;
 }
 
@@ -773,17 +784,23 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                         int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
                         int64_t ignore_index, int32_t use_ignore, hipStream_t stream)
 {
-    if (int rc = check_common(hidden, weight, N, H, V, dtype)) return rc;
+    if (int rc = check_common(N, H, V, dtype)) return rc;
     if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
-    if (!grad_logp || !targets || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (!grad_logp || !hidden || !weight || !targets || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
     if (!d_hidden && !d_weight && !d_bias) return rlk_fail(RLK_ERR_ARG, "no gradient requested");
     if (bias == nullptr && d_bias != nullptr) return rlk_fail(RLK_ERR_ARG, "d_bias given without bias");
     if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
     if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
-    const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
-    if (!workspace || workspace_bytes < p.total) return rlk_fail(RLK_ERR_ARG, "workspace too small");
+    size_t need = 0;
+    rlk_linear_logp_bwd_workspace_bytes(N, H, V, dtype, dz_budget_bytes, &need);
+    if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
     if (reinterpret_cast<uintptr_t>(workspace) & 255)
         return rlk_fail(RLK_ERR_ARG, "workspace must be 256-byte aligned");
+    if (!use_mfma(hidden, weight, H, dtype))
+        return generic_bwd(grad_logp, hidden, weight, bias, targets, lse, d_hidden, d_weight, d_bias,
+                           workspace, N, H, V, vocab_start, dtype, temperature, ignore_index,
+                           use_ignore, stream);
+    const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
 
     char* ws = static_cast<char*>(workspace);
     float* scales = reinterpret_cast<float*>(ws + p.scales_off);

@@ -17,7 +17,8 @@ import torch
 from .. import _native
 from ..platform import logger
 
-_DTYPES = {torch.bfloat16: _native.DTYPE_BF16, torch.float16: _native.DTYPE_F16}
+_DTYPES = {torch.bfloat16: _native.DTYPE_BF16, torch.float16: _native.DTYPE_F16,
+           torch.float32: _native.DTYPE_F32}
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -44,15 +45,15 @@ def _out_of_range_error(target_1d: torch.Tensor, vocab: int, ignore_index: Optio
     )
 
 
-def mfma_path_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
-    """bf16/f16 on the GPU with a hidden size the 16-byte tile loads can address."""
+def hip_path_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
+    """bf16 / f16 / f32 tensors of one dtype on one GPU.  bf16/f16 with a hidden size that is a
+    multiple of 8 run on the MFMA tiles, the rest on the scalar-FMA kernels (H <= 12288)."""
     return (
         hidden.is_cuda
         and weight.is_cuda
         and hidden.device == weight.device
         and hidden.dtype in _DTYPES
         and weight.dtype == hidden.dtype
-        and hidden.size(-1) % 8 == 0
     )
 
 
@@ -238,8 +239,9 @@ class RocmFusedLinearLogpOp:
         if global_vocab_size is not None and int(global_vocab_size) != vocab:
             raise ValueError("global_vocab_size differs from the local vocab size, but no "
                              "multi-rank tensor-parallel group was provided.")
-        if not mfma_path_supported(hidden, lm_head_weight):
+        if not hip_path_supported(hidden, lm_head_weight):
             raise NotImplementedError(
-                "RocmFusedLinearLogpOp: needs bf16/f16 CUDA tensors with hidden size % 8 == 0")
+                "RocmFusedLinearLogpOp needs hidden and lm_head_weight of one dtype "
+                "(bf16, f16 or f32) on the same GPU")
         return _FusedLinearLogpFunction.apply(hidden, lm_head_weight, bias, target_ids,
                                               float(temperature), ignore_index, check_targets)
