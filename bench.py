@@ -25,6 +25,12 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}  # MI355X dense MFMA, published
 
+# HBM bytes moved by ONE forward launch of the default workload, from two `rocprofv3 --pmc` runs of
+# this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
+# reads for the 1 GiB `--calibrate-copy` kernel (factors 2.000 and 1.000):
+# 2.000 * 25659100 KiB + 1.000 * 10752 KiB.  Other workloads report null.
+MEASURED_FWD_TRAFFIC_BYTES = {"llama3-8b-head": (2.0 * 25659100 + 10752) * 1024}
+
 WORKLOADS = {
     # BASELINE.json configs[1] shape; the metric is quoted on forward+backward at this shape
     "llama3-8b-head": dict(tokens=32768, hidden=4096, vocab=128256, dtype="bf16",
@@ -101,6 +107,9 @@ def main() -> int:
     ap.add_argument("--cpu-slice", type=int, default=1024,
                     help="tokens of the CPU-baseline slice (0 = skip the CPU baseline)")
     ap.add_argument("--mode", default="fwd+bwd", choices=["fwd+bwd", "fwd"])
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (known HBM traffic) so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -144,6 +153,13 @@ def main() -> int:
             out = (logp, lse, d_h, d_w)
         return out
 
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, device=dev, dtype=torch.float32)   # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        torch.neg(src, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     torch.cuda.synchronize()
     base_mem = torch.cuda.memory_allocated()
     torch.cuda.reset_peak_memory_stats()
@@ -200,7 +216,8 @@ def main() -> int:
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": None,
+            "traffic": MEASURED_FWD_TRAFFIC_BYTES.get(args.workload),
+            "algorithmic_bytes": float((n * h + v * h) * 2 + n * 8 + n * 8),
             "launch_ms": fwd_ms,
             "flops_per_launch": fwd_flops,
         },
