@@ -40,6 +40,18 @@ typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 #define RLK_ABLATE 0
 #endif
 
+// Main-loop variant: 1 = global memory is copied straight into LDS (no staging registers),
+// 0 = global -> registers -> LDS.  K steps that are not a whole BK always take the second.
+#ifndef RLK_DTL
+#define RLK_DTL 1
+#endif
+#ifndef RLK_LW
+#define RLK_LW 2  // direct-to-LDS: slices over which the loads of one K step are spread
+#endif
+#ifndef RLK_RD
+#define RLK_RD 8  // direct-to-LDS: fragment reads issued per 8 MFMA slots (8 = one per slot)
+#endif
+
 // Workgroup shape: kWM x kWN wavefronts tile the 256 x 256 block; each wavefront owns
 // kTM x kTN MFMA tiles of 32 x 32.
 #ifndef RLK_WM
@@ -247,6 +259,9 @@ __device__ inline void static_for(F&& f)
     }
 }
 
+template <class T, bool A_KMAJOR, bool B_KMAJOR, int BK>
+struct TileGemmDtl;
+
 // Workgroup tile contraction.  acc[i][j] (+)= A rows x B rows over k in [0, K).
 // smem must hold 2 * (A tile + B tile) bytes.  All 256 threads must call it (it barriers).
 //
@@ -392,10 +407,231 @@ struct TileGemm {
     __device__ static inline void run(const Operand& A, const Operand& B, int K,
                                       f32x16_t (&acc)[TM][TN], char* smem)
     {
-        if (K % BK == 0)
+        if (K % BK == 0) {
+#if RLK_DTL
+            TileGemmDtl<T, A_KMAJOR, B_KMAJOR, BK>::run(A, B, K, acc, smem);
+#else
             run_impl<false>(A, B, K, acc, smem);
-        else
+#endif
+        } else {
             run_impl<true>(A, B, K, acc, smem);
+        }
+    }
+};
+
+// ------------------------------------------------------------------------------------------- //
+// Direct-to-LDS variant of the main loop (used when K is a multiple of BK).
+//
+// Global memory is copied straight into LDS by `global_load_lds_dwordx4` (each lane's 16 bytes land
+// at M0 + lane * 16, so one wavefront instruction fills 1 KiB of consecutive LDS): no staging
+// registers, no LDS store instructions.  Because the destination is dense, bank conflicts are
+// avoided by an XOR swizzle applied on the GLOBAL side (which 16-byte chunk a lane fetches):
+//   K-contiguous tile, row r (128 B), chunk c      -> LDS  r*128 + ((c ^ ((r >> 1) & 7)) * 16)
+//   K-major tile,      k-line k (512 B), chunk c   -> LDS  k*512 + ((c ^ ((k & 3) << 2)) * 16)
+// which makes both the b128 fragment reads and the transposing b64 reads conflict-free.
+// Two LDS stages of BK = 64; the loads of K step kt+1 are issued during the last slice of step
+// kt-1 (right after the barrier that frees their buffer) and the first slices of step kt.
+// ------------------------------------------------------------------------------------------- //
+// s_waitcnt immediate that waits only for vmcnt <= n (expcnt and lgkmcnt left at "no wait").
+constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+template <bool KMAJOR, int ROWS, int BK>
+struct DtlIO {
+    static_assert(BK == 64 && ROWS == 256, "direct-to-LDS layout is written for 256 x 64 tiles");
+    static constexpr int kBytes = ROWS * BK * 2;            // 32 KiB, dense
+    static constexpr int kInstr = kBytes / 1024;            // wavefront loads per tile (32)
+    static constexpr int kWaves = kThreads / 64;
+    static constexpr int kPasses = kInstr / kWaves;         // loads per wavefront per K step
+    static_assert(kInstr % kWaves == 0, "loads must divide over the wavefronts");
+
+    const char* base;        // uniform: tile origin advanced to the current K step by the caller
+    uint32_t off[kPasses];   // per-lane byte offset of this lane's chunk for load p at K step 0
+    uint32_t step;           // uniform byte advance per K step
+    int wave;                // uniform wavefront index
+
+    __device__ inline void init(const Operand& op, int K)
+    {
+        const int lane = threadIdx.x & 63;
+        wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        base = reinterpret_cast<const char*>(op.base);
+        const uint32_t ld = static_cast<uint32_t>(op.ld);
+        step = KMAJOR ? static_cast<uint32_t>(BK) * ld * 2u : static_cast<uint32_t>(BK) * 2u;
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p) {
+            const int q = wave + kWaves * p;  // which 1 KiB block of the tile
+            if (KMAJOR) {
+                const int k = 2 * q + (lane >> 5);
+                const int c = (lane & 31) ^ ((k & 3) << 2);
+                const int kc = k < K ? k : K - 1;
+                const int r = c * 8 < op.rows ? c * 8 : 0;
+                off[p] = (static_cast<uint32_t>(kc) * ld + static_cast<uint32_t>(r)) * 2u;
+            } else {
+                const int r = 8 * q + (lane >> 3);
+                const int c = (lane & 7) ^ ((r >> 1) & 7);
+                const int rc = r < op.rows ? r : op.rows - 1;
+                off[p] = (static_cast<uint32_t>(rc) * ld + static_cast<uint32_t>(c * 8)) * 2u;
+            }
+        }
+    }
+
+    // Issue load p of K step kt into the tile at `lds` (uniform pointer).  Written as inline
+    // assembly (M0 = LDS destination, then the load with a scalar base and a 32-bit lane offset):
+    // the compiler then neither tracks the LDS write nor guards later LDS reads with vmcnt(0);
+    // the main loop waits explicitly (s_waitcnt vmcnt) before the barrier that publishes a stage.
+    __device__ inline void load_one(int kt, char* lds, int p) const
+    {
+        const char* src = base + static_cast<size_t>(kt) * step;  // uniform
+        const uint32_t dst = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+                                 (RLK_LDS char*)(lds))) + static_cast<uint32_t>((wave + kWaves * p) * 1024);
+        asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(off[p]), "s"(src), "s"(dst)
+                     : "memory", "m0");
+    }
+
+    // MFMA 32x32x16 operand fragment: lane l holds row (row0 + l%32), k = kk*16 + 8*(l/32) + 0..7.
+    __device__ static inline u32x4_t frag(const char* lds, int row0, int kk)
+    {
+        const int l = threadIdx.x & 63;
+        if (KMAJOR) {
+            const int a = (l & 15) >> 2;
+            const int b = l & 3;
+            const int kline = kk * 16 + 8 * (l >> 5) + a;           // kline & 3 == a
+            const int c = (row0 >> 3) + 2 * ((l >> 4) & 1) + (b >> 1);
+            const char* p0 = lds + kline * 512 + ((c ^ (a << 2)) * 16) + (b & 1) * 8;
+            const char* p1 = p0 + 4 * 512;                           // k-line + 4: same swizzle
+            s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RLK_LDS s16x4_t*)(p0));
+            s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RLK_LDS s16x4_t*)(p1));
+            u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
+            u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
+            return u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y};
+        } else {
+            const int r = row0 + (l & 31);
+            const int c = (2 * kk + (l >> 5)) ^ (((l & 31) >> 1) & 7);  // row0 is a multiple of 32
+            return *reinterpret_cast<const u32x4_t*>(lds + r * 128 + c * 16);
+        }
+    }
+};
+
+template <class T, bool A_KMAJOR, bool B_KMAJOR, int BK>
+struct TileGemmDtl {
+    static constexpr int TM = kTM;
+    static constexpr int TN = kTN;
+    static constexpr int KK = BK / 16;
+    using IOA = DtlIO<A_KMAJOR, 256, BK>;
+    using IOB = DtlIO<B_KMAJOR, 256, BK>;
+    static constexpr int PA = IOA::kPasses;
+    static constexpr int PB = IOB::kPasses;
+    static constexpr int NL = PA + PB;                 // loads per wavefront per K step
+    static constexpr int NM = TM * TN;                 // MFMAs per slice
+    static constexpr int LW = RLK_LW;                  // load window in slices
+    static_assert(LW >= 1 && LW <= KK - 1, "load window must end before the barrier slice");
+    static constexpr int kStageBytes = IOA::kBytes + IOB::kBytes;
+    static constexpr int kSmemBytes = 2 * kStageBytes;
+
+    // Load j of a K step is issued after MFMA slot j * (LW*NM) / NL of the window that starts at
+    // the last slice of the previous step.
+    template <int KKI>
+    __device__ static inline void slice(const IOA& la, const IOB& lb, u32x4_t (&fa)[2][TM],
+                                        u32x4_t (&fb)[2][TN], int wm, int wn, int kt, int nk,
+                                        char* cur, char* nxt, f32x16_t (&acc)[TM][TN])
+    {
+        constexpr bool last = KKI == KK - 1;
+        constexpr int setc = KKI & 1, setn = setc ^ 1;
+        constexpr int NR = TM + TN;
+        const char* rsrc = last ? nxt : cur;
+        constexpr int kkn = last ? 0 : KKI + 1;
+        // window slice index of this slice: the last slice opens the window of step kt+2
+        constexpr int wslice = last ? 0 : KKI + 1;
+        static_for<0, NM>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            constexpr int i = q / TN, j = q % TN;
+            acc[i][j] = T::mfma(fa[setc][i], fb[setc][j], acc[i][j]);
+            // fragment reads for the next slice: one per MFMA slot from the start of the slice, so
+            // that all of them have returned when the next slice begins
+            static_for<q * RLK_RD / 8, (q + 1) * RLK_RD / 8>([&](auto oc) {
+                constexpr int o = decltype(oc)::value;
+                if constexpr (o >= NR) {
+                } else if constexpr (o == 0 || o > TN) {
+                    constexpr int fi = o == 0 ? 0 : o - TN;
+                    fa[setn][fi] = IOA::frag(rsrc, wm * (TM * 32) + fi * 32, kkn);
+                } else {
+                    constexpr int fj = o - 1;
+                    fb[setn][fj] = IOB::frag(rsrc + IOA::kBytes, wn * (TN * 32) + fj * 32, kkn);
+                }
+            });
+            if constexpr (wslice < LW) {
+                constexpr int wslot = wslice * NM + q;
+                constexpr int lo = (wslot * NL + LW * NM - 1) / (LW * NM);        // ceil
+                constexpr int hi = ((wslot + 1) * NL + LW * NM - 1) / (LW * NM);  // ceil
+                static_for<lo, hi>([&](auto lc) {
+                    constexpr int g = decltype(lc)::value;
+                    // last slice: first loads of step kt+2 into the buffer this step just freed;
+                    // other slices: remaining loads of step kt+1 into the other buffer
+                    const int ks = last ? (kt + 2 < nk ? kt + 2 : nk - 1) : (kt + 1 < nk ? kt + 1 : nk - 1);
+                    char* dst = last ? cur : nxt;
+                    if constexpr (g < PA)
+                        la.load_one(ks, dst, g);
+                    else
+                        lb.load_one(ks, dst + IOA::kBytes, g - PA);
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    }
+
+    __device__ static inline void run(const Operand& A, const Operand& B, int K,
+                                      f32x16_t (&acc)[TM][TN], char* smem)
+    {
+        IOA la;
+        IOB lb;
+        u32x4_t fa[2][TM];
+        u32x4_t fb[2][TN];
+        const int wave = threadIdx.x >> 6;
+        const int wm = wave / kWN;
+        const int wn = wave % kWN;
+        la.init(A, K);
+        lb.init(B, K);
+        const int nk = K / BK;
+
+        // prologue: all of K step 0, and the part of K step 1 that a steady-state "last slice"
+        // would already have issued
+        static_for<0, PA>([&](auto pc) { la.load_one(0, smem, decltype(pc)::value); });
+        static_for<0, PB>([&](auto pc) { lb.load_one(0, smem + IOA::kBytes, decltype(pc)::value); });
+        {
+            constexpr int first = (NM * NL + LW * NM - 1) / (LW * NM);  // loads of window slice 0
+            const int k1 = nk > 1 ? 1 : 0;
+            static_for<0, first>([&](auto lc) {
+                constexpr int g = decltype(lc)::value;
+                if constexpr (g < PA)
+                    la.load_one(k1, smem + kStageBytes, g);
+                else
+                    lb.load_one(k1, smem + kStageBytes + IOA::kBytes, g - PA);
+            });
+            constexpr int wait_first = vmcnt_imm(first);
+            __builtin_amdgcn_s_waitcnt(wait_first);  // K step 0 has landed
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[0][i] = IOA::frag(smem, wm * (TM * 32) + i * 32, 0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            fb[0][j] = IOB::frag(smem + IOA::kBytes, wn * (TN * 32) + j * 32, 0);
+
+        for (int kt = 0; kt < nk; ++kt) {
+            char* cur = smem + (kt & 1) * kStageBytes;
+            char* nxt = smem + ((kt + 1) & 1) * kStageBytes;
+            static_for<0, KK - 1>([&](auto kc) {
+                slice<decltype(kc)::value>(la, lb, fa, fb, wm, wn, kt, nk, cur, nxt, acc);
+            });
+            constexpr int wait_all = vmcnt_imm(0);
+            __builtin_amdgcn_s_waitcnt(wait_all);  // my loads of K step kt+1 have landed
+            __syncthreads();
+            slice<KK - 1>(la, lb, fa, fb, wm, wn, kt, nk, cur, nxt, acc);
+        }
+        constexpr int wait_drain = vmcnt_imm(0);
+        __builtin_amdgcn_s_waitcnt(wait_drain);  // drain the re-fetches past the end
+        __syncthreads();                          // LDS may be reused by the caller
     }
 };
 
