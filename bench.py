@@ -28,8 +28,8 @@ PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}  # MI355X dense MFMA, published
 # HBM bytes moved by ONE forward launch of the default workload, from two `rocprofv3 --pmc` runs of
 # this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
 # reads for the 1 GiB `--calibrate-copy` kernel (factors 2.000 and 1.000):
-# 2.000 * 25659100 KiB + 1.000 * 10752 KiB.  Other workloads report null.
-MEASURED_FWD_TRAFFIC_BYTES = {"llama3-8b-head": (2.0 * 25659100 + 10752) * 1024}
+# 2.000 * 24915400 KiB + 1.000 * 4608 KiB.  Other workloads report null.
+MEASURED_FWD_TRAFFIC_BYTES = {"llama3-8b-head": (2.0 * 24915400 + 4608) * 1024}
 
 WORKLOADS = {
     # BASELINE.json configs[1] shape; the metric is quoted on forward+backward at this shape
@@ -39,6 +39,11 @@ WORKLOADS = {
                                temperature=0.7, ignore_frac=0.0),
     "qwen3-head": dict(tokens=131072, hidden=2048, vocab=151936, dtype="f16",
                        temperature=1.0, ignore_frac=0.01),
+    # BASELINE.json configs[4]: the configs[1] shape with the GRPO epilogue between forward and
+    # backward (one group of 64 responses x 512 positions, response lengths U{128..512})
+    "llama3-8b-grpo-step": dict(tokens=32768, hidden=4096, vocab=128256, dtype="bf16",
+                                temperature=1.0, ignore_frac=0.0, grpo=dict(group=64, seq=512,
+                                                                            clip_eps=0.2, beta=0.04)),
     "small": dict(tokens=4096, hidden=1024, vocab=32768, dtype="bf16", temperature=1.0,
                   ignore_frac=0.0),
 }
@@ -135,8 +140,45 @@ def main() -> int:
     do_bwd = args.mode == "fwd+bwd"
 
     fwd_ev = []
+    epi_ev = []
+    grpo = cfg.get("grpo")
+    if grpo:
+        from rl_kernel_amd.ops import grpo as GR
+
+        g, t = grpo["group"], grpo["seq"]
+        gen = torch.Generator(device=dev).manual_seed(1005)
+        lens = torch.randint(128, t + 1, (g,), device=dev, generator=gen)
+        mask = torch.arange(t, device=dev)[None, :] < lens[:, None]
+        targets = torch.where(mask.reshape(-1), targets, torch.full_like(targets, -100))
+        ign = -100
+        new_logp, _, _ = LL.fused_linear_logp_forward(hidden, weight, targets, None,
+                                                      temperature=temp, ignore_index=ign)
+        old = (new_logp + 0.05 * torch.randn(n, device=dev, generator=gen)).view(g, t)
+        ref = (new_logp + 0.05 * torch.randn(n, device=dev, generator=gen)).view(g, t)
+        rewards = torch.randn(g, device=dev, generator=gen)
+        del new_logp
+
+    def grpo_step(record):
+        logp, lse, _ = LL.fused_linear_logp_forward(hidden, weight, targets, None,
+                                                    temperature=temp, ignore_index=ign)
+        if record:
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+        adv = GR.group_advantages(rewards, samples_per_prompt=g)
+        out3, _, _, d_cur, _ = GR.grpo_from_logp_raw(logp.view(g, t), old, ref, adv, mask,
+                                                     clip_eps=grpo["clip_eps"], beta=grpo["beta"],
+                                                     want_grad=True)
+        if record:
+            e1.record()
+            epi_ev.append((e0, e1))
+        d_h, d_w, _ = LL.fused_linear_logp_backward(d_cur.reshape(-1), hidden, weight, targets, lse,
+                                                    None, temperature=temp, ignore_index=ign)
+        return (logp, lse, out3, d_h, d_w)
 
     def step(record=False):
+        if grpo:
+            return grpo_step(record)
         if record:
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
@@ -179,6 +221,17 @@ def main() -> int:
     ms = elapsed * 1e3 / args.steps
 
     deterministic = all(torch.equal(a, b) for a, b in zip(first, last))
+    if grpo:
+        # the forward launch is timed on its own after the steps (the step brackets the epilogue)
+        for _ in range(3):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            LL.fused_linear_logp_forward(hidden, weight, targets, None, temperature=temp,
+                                         ignore_index=ign)
+            e1.record()
+            fwd_ev.append((e0, e1))
+        torch.cuda.synchronize()
     fwd_ms = sum(a.elapsed_time(b) for a, b in fwd_ev) / len(fwd_ev)
     fwd_flops = 2.0 * n * h * v
     achieved = fwd_flops / (fwd_ms * 1e-3) / 1e12
@@ -222,6 +275,18 @@ def main() -> int:
             "flops_per_launch": fwd_flops,
         },
     }
+    if grpo:
+        epi_ms = sum(a.elapsed_time(b) for a, b in epi_ev) / len(epi_ev)
+        epi_bytes = n * (4 + 4 + 4 + 1 + 4 + 4)  # cur, old, ref, mask in; d_cur, d_kl out
+        result["metric"] = "GRPO step (logp fwd + loss epilogue + bwd) tokens/sec"
+        result["epilogue"] = {
+            "bound": "hbm", "ms": epi_ms, "algorithmic_bytes": epi_bytes,
+            "achieved": epi_bytes / (epi_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
+            "frac": epi_bytes / (epi_ms * 1e-3) / 1e9 / 8000.0,
+            "note": "group advantages + loss/grad launches incl. host launch gaps; 0.7 MB of "
+                    "traffic, launch-latency-bound",
+            "active_tokens": int(mask.sum().item()),
+        }
     if args.cpu_slice > 0:
         result["cpu_baseline"] = cpu_baseline(torch, cfg, args.cpu_slice)
     print(json.dumps(result))

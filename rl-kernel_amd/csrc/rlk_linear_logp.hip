@@ -560,10 +560,18 @@ struct FwdPlan {
     int total_splits;
 };
 
+#ifndef RLK_MIN_SPLIT
+#define RLK_MIN_SPLIT 4
+#endif
+
 int split_count(int row_blocks, int tiles)
 {
     if (tiles <= 0) return 0;
     int s = (512 + row_blocks / 2) / row_blocks;
+    // At least 4 splits when each still gets a long run of tiles: the 32 workgroups resident on
+    // one XCD then form an 8 x 4 (token blocks x splits) patch that fetches 12 distinct operand
+    // streams into its L2 instead of 18 (16 x 2) or 33 (32 x 1).
+    if (s < RLK_MIN_SPLIT && tiles >= RLK_MIN_SPLIT * 16) s = RLK_MIN_SPLIT;
     if (s < 1) s = 1;
     if (s > 64) s = 64;
     if (s > tiles) s = tiles;

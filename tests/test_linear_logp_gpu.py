@@ -263,3 +263,69 @@ def test_llama_head_shape_properties(dev):
     r_dh, _, _ = O.linear_logp_backward(gd[rows].cpu(), hd[rows].cpu(), wd.cpu(), td[rows].cpu(),
                                         ignore_index=-100)
     assert rel(d_h[rows], r_dh) < GRAD_REL
+
+
+@pytest.mark.parametrize("n,h,v,dtype,temp,ign_frac,seed", [
+    (65536, 4096, 128256, torch.bfloat16, 0.7, 0.0, 1003),    # BASELINE config 3
+    (131072, 2048, 151936, torch.float16, 1.0, 0.01, 1004),   # BASELINE config 4 (vocab tail tile)
+])
+def test_full_size_head_properties(dev, n, h, v, dtype, temp, ign_frac, seed):
+    """Full-size forward+backward: sampled token rows against the CPU oracle (logp, dH), exact
+    zeros on ignored rows, bitwise repeatability, zero column sums of dW, and sampled VOCAB rows
+    of dW (first, last -- inside the partial tail tile -- and a few between) recomputed on the
+    host in fp32 from the definition dW[v] = sum_n g_n/T (1[t_n = v] - exp(z_nv - lse_n)) H[n]."""
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    g = torch.Generator(device=dev).manual_seed(seed)
+    hd = torch.empty(n, h, device=dev, dtype=dtype)
+    for n0 in range(0, n, 16384):
+        hd[n0:n0 + 16384] = torch.randn(min(16384, n - n0), h, device=dev, generator=g).to(dtype)
+    wd = torch.empty(v, h, device=dev, dtype=dtype)
+    for v0 in range(0, v, 16384):
+        v1 = min(v, v0 + 16384)
+        wd[v0:v1] = (torch.randn(v1 - v0, h, device=dev, generator=g) * 0.02).to(dtype)
+    td = torch.randint(0, v, (n,), device=dev, generator=g)
+    ignored = torch.rand(n, device=dev, generator=g) < ign_frac
+    td[ignored] = -100
+    gd = torch.randn(n, device=dev, generator=g)
+    ign = -100 if ign_frac > 0 else None
+
+    logp, lse, err = LL.fused_linear_logp_forward(hd, wd, td, temperature=temp, ignore_index=ign)
+    logp2, lse2, _ = LL.fused_linear_logp_forward(hd, wd, td, temperature=temp, ignore_index=ign)
+    assert int(err.item()) == 0
+    assert torch.equal(logp, logp2) and torch.equal(lse, lse2)
+    assert torch.equal(logp[ignored], torch.zeros_like(logp[ignored]))
+    rows = torch.arange(3, n, n // 16)[:16]
+    if ign_frac > 0:
+        rows = torch.cat([rows, ignored.nonzero().flatten()[:4].cpu()])
+    w_cpu = wd.cpu()
+    ref, ref_lse = O.linear_logp(hd[rows].cpu(), w_cpu, td[rows].cpu(), temperature=temp,
+                                 ignore_index=ign, return_lse=True)
+    assert (logp[rows].cpu() - ref).abs().max().item() < LOGP_ATOL
+    assert (lse[rows].cpu() - ref_lse).abs().max().item() < LOGP_ATOL
+
+    d_h, d_w, _ = LL.fused_linear_logp_backward(gd, hd, wd, td, lse, temperature=temp,
+                                                ignore_index=ign)
+    d_h2, d_w2, _ = LL.fused_linear_logp_backward(gd, hd, wd, td, lse, temperature=temp,
+                                                  ignore_index=ign)
+    assert torch.equal(d_h, d_h2) and torch.equal(d_w, d_w2)
+    del d_h2, d_w2
+    assert torch.equal(d_h[ignored], torch.zeros_like(d_h[ignored]))
+    assert torch.isfinite(d_w).all() and torch.isfinite(d_h).all()
+    col_sum = d_w.sum(dim=0)
+    scale = d_w.abs().sum(dim=0)
+    assert (col_sum.abs() / scale.clamp_min(1e-20)).max().item() < 5e-3
+    r_dh, _, _ = O.linear_logp_backward(gd[rows].cpu(), hd[rows].cpu(), w_cpu, td[rows].cpu(),
+                                        temperature=temp, ignore_index=ign)
+    assert rel(d_h[rows], r_dh) < GRAD_REL
+
+    vrows = torch.tensor([0, 255, 256, v // 2 + 17, v - 257, v - 2, v - 1])
+    h_cpu = hd.cpu().float()
+    z = h_cpu @ w_cpu[vrows].float().t() / temp                       # [n, 7]
+    t_cpu, lse_cpu, g_cpu = td.cpu(), lse.cpu(), gd.cpu()
+    dz = -(z - lse_cpu[:, None]).exp()
+    dz += (t_cpu[:, None] == vrows[None, :]).float()
+    dz *= (g_cpu / temp)[:, None]
+    dz[t_cpu == -100] = 0.0
+    ref_dw = dz.t() @ h_cpu
+    assert rel(d_w[vrows], ref_dw) < GRAD_REL
