@@ -570,7 +570,8 @@ struct TileGemmDtl {
                     // other slices: remaining loads of step kt+1 into the other buffer
                     const int ks = last ? (kt + 2 < nk ? kt + 2 : nk - 1) : (kt + 1 < nk ? kt + 1 : nk - 1);
                     char* dst = last ? cur : nxt;
-                    if constexpr (g < PA)
+                    if constexpr ((RLK_ABLATE & 64) != 0) {  // dev: time without global loads
+                    } else if constexpr (g < PA)
                         la.load_one(ks, dst, g);
                     else
                         lb.load_one(ks, dst + IOA::kBytes, g - PA);

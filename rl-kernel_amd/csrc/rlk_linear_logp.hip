@@ -272,6 +272,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     Gemm::run(A, B, a.H, acc, smem);
+    if constexpr ((RLK_ABLATE & 32) != 0) { if (a.tok_valid >= 0) return; }  // dev: time without epilogue
 
     const float gscale = a.scales[0];
     const int vw = v0 + wm * (TM * 32);
@@ -359,6 +360,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     Gemm::run(A, B, a.v_valid, acc, smem);
+    if constexpr ((RLK_ABLATE & 32) != 0) { if (a.tok_valid >= 0) return; }  // dev: time without epilogue
 
     // Epilogue: all reads of the running fp32 partial are issued before the first use (clamped
     // addresses instead of branches), then added and stored under a predicate.
@@ -441,6 +443,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     Gemm::run(A, B, a.tok_valid, acc, smem);
+    if constexpr ((RLK_ABLATE & 32) != 0) { if (a.tok_valid >= 0) return; }  // dev: time without epilogue
 
     // Epilogue: read-modify-write of the fp32 dW tile; the 16 reads of one MFMA tile are issued
     // together (clamped addresses), then added and stored under a predicate.
