@@ -112,6 +112,8 @@ def main() -> int:
     ap.add_argument("--cpu-slice", type=int, default=1024,
                     help="tokens of the CPU-baseline slice (0 = skip the CPU baseline)")
     ap.add_argument("--mode", default="fwd+bwd", choices=["fwd+bwd", "fwd"])
+    ap.add_argument("--dtype", default=None, choices=["bf16", "f16"],
+                    help="override the workload's 16-bit input type")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known HBM traffic) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
@@ -130,7 +132,9 @@ def main() -> int:
 
     from rl_kernel_amd.ops import linear_logp as LL
 
-    cfg = WORKLOADS[args.workload]
+    cfg = dict(WORKLOADS[args.workload])
+    if args.dtype:
+        cfg["dtype"] = args.dtype
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     hidden, weight, targets, grad = make_inputs(torch, cfg, dev)

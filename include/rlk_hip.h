@@ -95,13 +95,20 @@ int rlk_linear_logp_fwd(const void* hidden, const void* weight, const float* bia
  *   d_weight = dZ^T H    (f32, overwritten)
  *   d_bias   = sum_n dZ  (f32, only when bias != NULL)
  * dZ only ever exists as one (token chunk) x (vocab piece) block of at most `dz_budget_bytes`
- * (0 = default 512 MiB) inside `workspace`, so extra memory does not grow with N.
+ * (0 = default 256 MiB) inside `workspace`, so extra memory does not grow with N.
  * `lse` must be the natural-log logsumexp over the FULL vocabulary (for a shard: after the
  * cross-shard merge).  Any of d_hidden / d_weight / d_bias may be NULL to skip that gradient
  * (d_bias requires bias).
  * ------------------------------------------------------------------------------------------ */
 int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                         size_t dz_budget_bytes, size_t* bytes);
+
+/* Schedule the backward will use for these sizes (no counterpart in the reference, whose chunk is
+ * fixed at 2^24 / V tokens, rl_engine/kernels/ops/pytorch/loss/linear_logp.py:398-400):
+ * out4 = { tokens per chunk, vocab rows per piece, number of chunks, number of pieces }.  Host
+ * only; touches no device. */
+int rlk_linear_logp_bwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                             size_t dz_budget_bytes, int64_t* out4);
 
 int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* weight,
                         const float* bias, const int64_t* targets, const float* lse,

@@ -11,7 +11,7 @@
 #endif
 
 #ifndef RLK_DEFAULT_DZ_BUDGET
-#define RLK_DEFAULT_DZ_BUDGET (static_cast<size_t>(512) << 20)  // bytes of one dZ block
+#define RLK_DEFAULT_DZ_BUDGET (static_cast<size_t>(256) << 20)  // bytes of one dZ block
 #endif
 
 // Records `msg` as the calling thread's last error and returns `code` (always negative).

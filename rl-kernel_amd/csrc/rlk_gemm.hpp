@@ -36,6 +36,9 @@ typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 
 // Development switch for timing experiments (wrong results when non-zero): bit 0 drops the
 // global loads of the main loop, bit 1 the LDS stores, bit 2 the fragment reads, bit 3 the barrier.
+#ifndef RLK_STREAM
+#define RLK_STREAM 1  // 1: forward and dZ run all tiles of a workgroup through one pipeline
+#endif
 #ifndef RLK_ABLATE
 #define RLK_ABLATE 0
 #endif
@@ -444,9 +447,11 @@ struct DtlIO {
     static constexpr int kPasses = kInstr / kWaves;         // loads per wavefront per K step
     static_assert(kInstr % kWaves == 0, "loads must divide over the wavefronts");
 
-    const char* base;        // uniform: tile origin advanced to the current K step by the caller
+    const char* base;        // uniform: origin of the current tile
+    const char* next;        // uniform: origin of the tile whose first K steps follow this one's
     uint32_t off[kPasses];   // per-lane byte offset of this lane's chunk for load p at K step 0
     uint32_t step;           // uniform byte advance per K step
+    int nk;                  // K steps per tile
     int wave;                // uniform wavefront index
 
     __device__ inline void init(const Operand& op, int K)
@@ -454,6 +459,10 @@ struct DtlIO {
         const int lane = threadIdx.x & 63;
         wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
         base = reinterpret_cast<const char*>(op.base);
+        next = base;
+        nk = K / BK;
+        next = base;
+        nk = K / BK;
         const uint32_t ld = static_cast<uint32_t>(op.ld);
         step = KMAJOR ? static_cast<uint32_t>(BK) * ld * 2u : static_cast<uint32_t>(BK) * 2u;
 #pragma unroll
@@ -480,7 +489,11 @@ struct DtlIO {
     // the main loop waits explicitly (s_waitcnt vmcnt) before the barrier that publishes a stage.
     __device__ inline void load_one(int kt, char* lds, int p) const
     {
-        const char* src = base + static_cast<size_t>(kt) * step;  // uniform
+        if constexpr ((RLK_ABLATE & 128) != 0) kt &= 1;  // dev: every K step re-reads cached lines
+        // K steps past the end of this tile are the first steps of the next one (all uniform)
+        const bool over = kt >= nk;
+        const int rel = over ? (kt - nk < nk ? kt - nk : nk - 1) : kt;
+        const char* src = (over ? next : base) + static_cast<size_t>(rel) * step;
         const uint32_t dst = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
                                  (RLK_LDS char*)(lds))) + static_cast<uint32_t>((wave + kWaves * p) * 1024);
         asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
@@ -568,7 +581,7 @@ struct TileGemmDtl {
                     constexpr int g = decltype(lc)::value;
                     // last slice: first loads of step kt+2 into the buffer this step just freed;
                     // other slices: remaining loads of step kt+1 into the other buffer
-                    const int ks = last ? (kt + 2 < nk ? kt + 2 : nk - 1) : (kt + 1 < nk ? kt + 1 : nk - 1);
+                    const int ks = last ? kt + 2 : kt + 1;  // past the end = next tile (load_one)
                     char* dst = last ? cur : nxt;
                     if constexpr ((RLK_ABLATE & 64) != 0) {  // dev: time without global loads
                     } else if constexpr (g < PA)
@@ -581,58 +594,92 @@ struct TileGemmDtl {
         });
     }
 
-    __device__ static inline void run(const Operand& A, const Operand& B, int K,
-                                      f32x16_t (&acc)[TM][TN], char* smem)
-    {
+    // Pipeline state that lives across the tiles one workgroup computes back to back: the K loop
+    // of a tile fetches the first K steps of the next tile where it would otherwise run dry, so
+    // only the first tile of a workgroup pays the fill latency.
+    struct Stream {
         IOA la;
         IOB lb;
         u32x4_t fa[2][TM];
         u32x4_t fb[2][TN];
-        const int wave = threadIdx.x >> 6;
-        const int wm = wave / kWN;
-        const int wn = wave % kWN;
-        la.init(A, K);
-        lb.init(B, K);
-        const int nk = K / BK;
+        int wm, wn, nk, phase;
+    };
 
-        // prologue: all of K step 0, and the part of K step 1 that a steady-state "last slice"
-        // would already have issued
-        static_for<0, PA>([&](auto pc) { la.load_one(0, smem, decltype(pc)::value); });
-        static_for<0, PB>([&](auto pc) { lb.load_one(0, smem + IOA::kBytes, decltype(pc)::value); });
-        {
-            constexpr int first = (NM * NL + LW * NM - 1) / (LW * NM);  // loads of window slice 0
-            const int k1 = nk > 1 ? 1 : 0;
-            static_for<0, first>([&](auto lc) {
-                constexpr int g = decltype(lc)::value;
-                if constexpr (g < PA)
-                    la.load_one(k1, smem + kStageBytes, g);
-                else
-                    lb.load_one(k1, smem + kStageBytes + IOA::kBytes, g - PA);
-            });
-            constexpr int wait_first = vmcnt_imm(first);
-            __builtin_amdgcn_s_waitcnt(wait_first);  // K step 0 has landed
-        }
+    // Fill the pipeline for the first tile: K step 0 in LDS and published, the fragments of its
+    // first slice in registers, the head of K step 1 in flight.
+    __device__ static inline void begin(Stream& st, const Operand& A, const Operand& B, int K,
+                                        char* smem)
+    {
+        const int wave = threadIdx.x >> 6;
+        st.wm = wave / kWN;
+        st.wn = wave % kWN;
+        st.la.init(A, K);
+        st.lb.init(B, K);
+        st.nk = K / BK;
+        st.phase = 0;
+        static_for<0, PA>([&](auto pc) { st.la.load_one(0, smem, decltype(pc)::value); });
+        static_for<0, PB>(
+            [&](auto pc) { st.lb.load_one(0, smem + IOA::kBytes, decltype(pc)::value); });
+        constexpr int first = (NM * NL + LW * NM - 1) / (LW * NM);  // loads of window slice 0
+        static_for<0, first>([&](auto lc) {
+            constexpr int g = decltype(lc)::value;
+            if constexpr (g < PA)
+                st.la.load_one(1, smem + kStageBytes, g);
+            else
+                st.lb.load_one(1, smem + kStageBytes + IOA::kBytes, g - PA);
+        });
+        constexpr int wait_first = vmcnt_imm(first);
+        __builtin_amdgcn_s_waitcnt(wait_first);  // K step 0 has landed
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[0][i] = IOA::frag(smem, wm * (TM * 32) + i * 32, 0);
+        for (int i = 0; i < TM; ++i) st.fa[0][i] = IOA::frag(smem, st.wm * (TM * 32) + i * 32, 0);
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-            fb[0][j] = IOB::frag(smem + IOA::kBytes, wn * (TN * 32) + j * 32, 0);
+            st.fb[0][j] = IOB::frag(smem + IOA::kBytes, st.wn * (TN * 32) + j * 32, 0);
+    }
 
+    // All K steps of the current tile into `acc`.  `next_a` / `next_b` are the operand origins of
+    // the tile that follows (same leading dimensions and row counts; pass the current origins
+    // after the last tile: the extra fetches then stay inside the same tile).  On return the
+    // stream stands at the start of that tile exactly as begin() leaves it.
+    __device__ static inline void tile(Stream& st, const void* next_a, const void* next_b,
+                                       f32x16_t (&acc)[TM][TN], char* smem)
+    {
+        st.la.next = reinterpret_cast<const char*>(next_a);
+        st.lb.next = reinterpret_cast<const char*>(next_b);
+        const int nk = st.nk;
         for (int kt = 0; kt < nk; ++kt) {
-            char* cur = smem + (kt & 1) * kStageBytes;
-            char* nxt = smem + ((kt + 1) & 1) * kStageBytes;
+            char* cur = smem + ((kt + st.phase) & 1) * kStageBytes;
+            char* nxt = smem + ((kt + st.phase + 1) & 1) * kStageBytes;
             static_for<0, KK - 1>([&](auto kc) {
-                slice<decltype(kc)::value>(la, lb, fa, fb, wm, wn, kt, nk, cur, nxt, acc);
+                slice<decltype(kc)::value>(st.la, st.lb, st.fa, st.fb, st.wm, st.wn, kt, nk, cur,
+                                           nxt, acc);
             });
             constexpr int wait_all = vmcnt_imm(0);
             __builtin_amdgcn_s_waitcnt(wait_all);  // my loads of K step kt+1 have landed
             __syncthreads();
-            slice<KK - 1>(la, lb, fa, fb, wm, wn, kt, nk, cur, nxt, acc);
+            slice<KK - 1>(st.la, st.lb, st.fa, st.fb, st.wm, st.wn, kt, nk, cur, nxt, acc);
         }
+        st.phase = (st.phase + nk) & 1;
+        st.la.base = st.la.next;
+        st.lb.base = st.lb.next;
+    }
+
+    // Drain the fetches issued for a tile that will not be computed; LDS is free afterwards.
+    __device__ static inline void end(Stream&)
+    {
         constexpr int wait_drain = vmcnt_imm(0);
-        __builtin_amdgcn_s_waitcnt(wait_drain);  // drain the re-fetches past the end
-        __syncthreads();                          // LDS may be reused by the caller
+        __builtin_amdgcn_s_waitcnt(wait_drain);
+        __syncthreads();
+    }
+
+    __device__ static inline void run(const Operand& A, const Operand& B, int K,
+                                      f32x16_t (&acc)[TM][TN], char* smem)
+    {
+        Stream st;
+        begin(st, A, B, K, smem);
+        tile(st, A.base, B.base, acc, smem);
+        end(st);
     }
 };
 

@@ -7,6 +7,8 @@
 // forward and in the dZ recompute M = vocab and N = token, so one lane owns whole token columns
 // and the softmax reduction over vocab is a plain in-register loop with no cross-lane traffic.
 #include "rlk_common.hpp"
+#include <vector>
+
 #include "rlk_gemm.hpp"
 
 namespace rlk {
@@ -72,15 +74,27 @@ __device__ inline void fwd_epilogue(const f32x16_t (&acc)[kTM][kTN], const FwdAr
         const int etgt = (static_cast<unsigned>(tl) < static_cast<unsigned>(kTM * 32) && ((x >> 2) & 1) == (lane >> 5))
                              ? ((tl >> 5) * 16 + (x >> 3) * 4 + (x & 3))
                              : -1;
-        float sum = 0.f, zraw = 0.f;
+        // four partial sums (fixed association) keep the exp results off a single add chain; the
+        // target capture runs only when some lane of the wavefront owns a target row in this slab
+        float ps[4] = {0.f, 0.f, 0.f, 0.f};
+        float zraw = 0.f;
+        if (__builtin_amdgcn_ballot_w64(etgt >= 0) != 0) {  // uniform
 #pragma unroll
-        for (int i = 0; i < kTM; ++i)
+            for (int i = 0; i < kTM; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float z = logit(i, j, r);
-                sum += __builtin_amdgcn_exp2f(fmaf(z, a.scale2, -mref));
-                zraw = (etgt == i * 16 + r) ? z : zraw;
-            }
+                for (int r = 0; r < 16; ++r) {
+                    const float z = logit(i, j, r);
+                    ps[r & 3] += __builtin_amdgcn_exp2f(fmaf(z, a.scale2, -mref));
+                    zraw = (etgt == i * 16 + r) ? z : zraw;
+                }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kTM; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    ps[r & 3] += __builtin_amdgcn_exp2f(fmaf(logit(i, j, r), a.scale2, -mref));
+        }
+        const float sum = (ps[0] + ps[1]) + (ps[2] + ps[3]);
         __builtin_amdgcn_sched_barrier(0);
         s[j] = s[j] * __builtin_amdgcn_exp2f(m[j] - mref) + sum;
         m[j] = mnew;
@@ -124,18 +138,39 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
     }
 
     Operand B{a.hidden + static_cast<int64_t>(tok0) * a.H, a.H, tok_valid};
-    for (int vt = t0; vt < t1; ++vt) {
-        const int v0 = vt * 256;
-        Operand A{a.weight + static_cast<int64_t>(v0) * a.H, a.H, min(256, a.V - v0)};
-        f32x16_t acc[TM][TN];
+    auto tile_origin = [&](int vt) { return a.weight + static_cast<int64_t>(vt) * 256 * a.H; };
+    if (!GENERAL && RLK_DTL != 0 && RLK_STREAM != 0 && a.H % BK == 0 && t0 < t1) {
+        // every tile is full: one pipeline runs through all tiles of the range, the K loop of a
+        // tile already fetching the head of the next one while the softmax update runs
+        using Dtl = TileGemmDtl<T, false, false, BK>;
+        typename Dtl::Stream st;
+        Dtl::begin(st, Operand{tile_origin(t0), a.H, 256}, B, a.H, smem);
+        for (int vt = t0; vt < t1; ++vt) {
+            f32x16_t acc[TM][TN];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+                for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-        Gemm::run(A, B, a.H, acc, smem);
-        fwd_epilogue<GENERAL>(acc, a, v0 + wm * (TM * 32), lane, tgt, m, s, zt);
+                    for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            Dtl::tile(st, tile_origin(vt + 1 < t1 ? vt + 1 : vt), B.base, acc, smem);
+            fwd_epilogue<GENERAL>(acc, a, vt * 256 + wm * (TM * 32), lane, tgt, m, s, zt);
+        }
+        Dtl::end(st);
+    } else {
+        for (int vt = t0; vt < t1; ++vt) {
+            const int v0 = vt * 256;
+            Operand A{tile_origin(vt), a.H, min(256, a.V - v0)};
+            f32x16_t acc[TM][TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            Gemm::run(A, B, a.H, acc, smem);
+            fwd_epilogue<GENERAL>(acc, a, v0 + wm * (TM * 32), lane, tgt, m, s, zt);
+        }
     }
 
     // Merge the two half-wave row groups (same token, different vocab rows), then the two
@@ -245,6 +280,10 @@ struct DzArgs {
     float scale2;
 };
 
+// Row pitch of the dZ tile staged in LDS: 512 bytes of data + 8, so that the 32 lanes of a half
+// wavefront (32 tokens, same vocab column) write 8 bytes each into distinct bank pairs.
+constexpr int kDzPitch = 520;
+
 // GENERAL = false: no bias, every vocab tile of the launch is full.
 template <class T, int BK, bool GENERAL>
 __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
@@ -271,6 +310,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    static_assert(256 * kDzPitch <= Gemm::kSmemBytes, "staged dZ tile must fit the GEMM's LDS");
     Gemm::run(A, B, a.H, acc, smem);
     if constexpr ((RLK_ABLATE & 32) != 0) { if (a.tok_valid >= 0) return; }  // dev: time without epilogue
 
@@ -291,7 +331,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
         const int etgt = (tr >= 0 && ((x >> 2) & 1) == (lane >> 5))
                              ? ((tr >> 5) * 16 + (x >> 3) * 4 + (x & 3))
                              : -1;
-        uint16_t* drow = a.dz + static_cast<int64_t>(tok0 + tl) * a.ldz + vw + 4 * (lane >> 5);
+        // the 16-bit tile is staged in LDS as [token][vocab] rows so that it leaves in full lines
+        char* srow = smem + tl * kDzPitch + (wm * (TM * 32) + 4 * (lane >> 5)) * 2;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -313,8 +354,20 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
                     o[c] = T::from_float(fmaf(-gs, p, hit));
                 }
                 u32x2_t pk{o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
-                *reinterpret_cast<u32x2_t*>(drow + i * 32 + 8 * q) = pk;
+                *reinterpret_cast<u32x2_t*>(srow + (i * 32 + 8 * q) * 2) = pk;
             }
+    }
+    __syncthreads();
+    // copy-out: a half wavefront moves one 512-byte row (4 full lines), 16 bytes per lane
+    uint16_t* dtile = a.dz + static_cast<int64_t>(tok0) * a.ldz + v0;
+#pragma unroll 4
+    for (int it = 0; it < 256 / (2 * (kThreads / 64)); ++it) {
+        const int row = it * (2 * (kThreads / 64)) + 2 * wave + (lane >> 5);
+        const char* src = smem + row * kDzPitch + (lane & 31) * 16;  // 8-byte aligned (pitch)
+        const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(src);
+        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(src + 8);
+        *reinterpret_cast<u32x4_t*>(dtile + static_cast<int64_t>(row) * a.ldz + (lane & 31) * 8) =
+            u32x4_t{lo.x, lo.y, hi.x, hi.y};
     }
 }
 
@@ -607,28 +660,84 @@ struct BwdPlan {
     size_t scales_off, dz_off, acc_off, total;
 };
 
-// Balanced token chunks / vocab pieces so that one dZ block stays within `budget` bytes.
+// Cost of the three launches of one dZ block of ct x pt tiles, in K steps of one CU: a launch of
+// t tiles occupies ceil(t / 256) rounds of the 256 CUs, a tile costs its K steps plus an epilogue
+// (dZ: exp + 16-bit store; dH / dW: fp32 read-modify-write of the tile).
+inline int64_t block_cost(int64_t ct, int64_t pt, int64_t ht, int64_t hk)
+{
+    const int64_t dz = (ct * pt + 255) / 256 * (hk + 12);
+    const int64_t dh = (ct * ht + 255) / 256 * (4 * pt + 28);
+    const int64_t dw = (pt * ht + 255) / 256 * (4 * ct + 28);
+    return dz + dh + dw;
+}
+
+// Token chunks x vocab pieces such that one dZ block stays within `budget` bytes and block plus
+// fp32 dH accumulator within 1.5 x budget.  Among the shapes that fit, the one with the lowest
+// modelled time wins: tile counts just above a multiple of 256 waste most of a round, and small
+// blocks pay the read-modify-write epilogues more often.
 BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
 {
-    BwdPlan p;
+    struct Key {
+        int64_t N, V;
+        int H;
+        size_t budget;
+        BwdPlan plan;
+    };
+    static thread_local Key memo{0, 0, 0, 0, {}};
+    if (memo.N == N && memo.V == V && memo.H == H && memo.budget == budget) return memo.plan;
+
     const int64_t n_t = (N + 255) / 256, v_t = (V + 255) / 256;
-    // square-ish block: side (in tiles) so that side^2 * 256*256*2 <= budget
-    int64_t side = 1;
-    while ((side + 1) * (side + 1) * 131072 <= static_cast<int64_t>(budget)) ++side;
-    int64_t ct = n_t < side ? n_t : side;
-    int64_t pt = static_cast<int64_t>(budget) / (ct * 131072);
-    if (pt > v_t) pt = v_t;
-    if (pt < 1) pt = 1;
-    p.n_chunks = static_cast<int>((n_t + ct - 1) / ct);
-    p.n_pieces = static_cast<int>((v_t + pt - 1) / pt);
-    p.tok_chunk = static_cast<int>((n_t + p.n_chunks - 1) / p.n_chunks) * 256;
-    p.v_piece = static_cast<int>((v_t + p.n_pieces - 1) / p.n_pieces) * 256;
+    const int64_t ht = (H + 255) / 256, hk = (H + kBK - 1) / kBK;
+    const int64_t tile_bytes = 131072;                          // 256 x 256 16-bit
+    const int64_t max_tiles = static_cast<int64_t>(budget) / tile_bytes;
+    const int64_t cap = static_cast<int64_t>(budget) + static_cast<int64_t>(budget) / 2;
+
+    // candidate sizes: balanced splits ceil(x / k) and multiples of 8 tiles
+    auto candidates = [](int64_t x, std::vector<int64_t>& out) {
+        for (int64_t k = 1; k <= x; ++k) {
+            const int64_t c = (x + k - 1) / k;
+            if (out.empty() || out.back() != c) out.push_back(c);
+        }
+        for (int64_t c = 8; c <= x; c += 8) out.push_back(c);
+    };
+    std::vector<int64_t> cts, pts;
+    candidates(n_t, cts);
+    candidates(v_t, pts);
+
+    int64_t best_ct = 1, best_pt = 1, best_cost = -1, best_bytes = 0;
+    for (int64_t ct : cts) {
+        if (ct > max_tiles) continue;
+        const int64_t nc = (n_t + ct - 1) / ct, ct_last = n_t - (nc - 1) * ct;
+        for (int64_t pt : pts) {
+            if (ct * pt > max_tiles) continue;
+            const int64_t np = (v_t + pt - 1) / pt, pt_last = v_t - (np - 1) * pt;
+            const int64_t bytes = ct * pt * tile_bytes + (np > 1 ? ct * 256 * H * 4 : 0);
+            if (bytes > cap && ct * pt > 1) continue;
+            const int64_t cost = (nc - 1) * (np - 1) * block_cost(ct, pt, ht, hk) +
+                                 (np - 1) * block_cost(ct_last, pt, ht, hk) +
+                                 (nc - 1) * block_cost(ct, pt_last, ht, hk) +
+                                 block_cost(ct_last, pt_last, ht, hk);
+            if (best_cost < 0 || cost < best_cost || (cost == best_cost && bytes < best_bytes)) {
+                best_cost = cost;
+                best_ct = ct;
+                best_pt = pt;
+                best_bytes = bytes;
+            }
+        }
+    }
+
+    BwdPlan p;
+    p.tok_chunk = static_cast<int>(best_ct) * 256;
+    p.v_piece = static_cast<int>(best_pt) * 256;
+    p.n_chunks = static_cast<int>((n_t + best_ct - 1) / best_ct);
+    p.n_pieces = static_cast<int>((v_t + best_pt - 1) / best_pt);
     p.dz_bytes = static_cast<size_t>(p.tok_chunk) * p.v_piece * 2;
     p.acc_bytes = p.n_pieces > 1 ? static_cast<size_t>(p.tok_chunk) * H * 4 : 0;
     p.scales_off = 0;
     p.dz_off = 256;
     p.acc_off = p.dz_off + align_up(p.dz_bytes, 256);
     p.total = p.acc_off + align_up(p.acc_bytes, 256);
+    memo = Key{N, V, H, budget, p};
     return p;
 }
 
@@ -785,6 +894,21 @@ int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t
     // large enough for either implementation (the choice also depends on pointer alignment)
     const size_t a = bwd_plan(N, H, V, dz_budget_bytes).total, b = generic_bwd_workspace(N, H, V);
     *bytes = a > b ? a : b;
+    return 0;
+}
+
+int rlk_linear_logp_bwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype, size_t dz_budget_bytes,
+                             int64_t* out4)
+{
+    (void)dtype;
+    if (!out4 || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad plan query");
+    if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
+    if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
+    const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
+    out4[0] = p.tok_chunk;
+    out4[1] = p.v_piece;
+    out4[2] = p.n_chunks;
+    out4[3] = p.n_pieces;
     return 0;
 }
 

@@ -45,18 +45,38 @@ def test_binding_covers_every_declared_symbol(native):
     assert lib.rlk_last_error() is not None
 
 
-def test_backward_workspace_is_constant_in_token_count(native):
+def _plan(lib, n, h, v, dtype=0, budget=0):
+    out = (ctypes.c_int64 * 4)()
+    assert lib.rlk_linear_logp_bwd_plan(n, h, v, dtype, budget, out) == 0
+    return tuple(out)
+
+
+def test_backward_workspace_is_bounded_in_token_count(native):
     lib = native.load()
     sizes = []
-    for n in (32768, 65536, 131072, 262144):
+    for n in (32768, 65536, 131072, 262144, 1 << 20):
         need = ctypes.c_size_t(0)
         assert lib.rlk_linear_logp_bwd_workspace_bytes(n, 4096, 128256, 0, 0, ctypes.byref(need)) == 0
         sizes.append(need.value)
-    assert len(set(sizes)) == 1, sizes          # same scratch for G = 64, 128, 256, 512
-    assert sizes[0] <= 1 << 30                  # <= 1 GiB extra HBM
+    # scratch does not grow with G = 64 ... 2048: one dZ block (<= 256 MiB) + fp32 dH chunk
+    assert max(sizes) <= (384 << 20) + 4096, sizes
+    assert max(sizes) <= 1 << 30                # <= 1 GiB extra HBM
     need = ctypes.c_size_t(0)
     assert lib.rlk_linear_logp_bwd_workspace_bytes(131072, 2048, 151936, 1, 0, ctypes.byref(need)) == 0
     assert need.value <= 1 << 30
+
+
+@pytest.mark.parametrize("n,h,v", [(32768, 4096, 128256), (65536, 4096, 128256),
+                                   (131072, 2048, 151936), (300, 64, 1000), (1 << 20, 4096, 128256)])
+@pytest.mark.parametrize("budget", [0, 64 << 20, 1 << 30])
+def test_backward_plan_covers_the_problem_within_budget(native, n, h, v, budget):
+    lib = native.load()
+    tok_chunk, v_piece, n_chunks, n_pieces = _plan(lib, n, h, v, 0, budget)
+    assert tok_chunk % 256 == 0 and v_piece % 256 == 0 and tok_chunk > 0 and v_piece > 0
+    assert tok_chunk * n_chunks >= n > tok_chunk * (n_chunks - 1)
+    assert v_piece * n_pieces >= v > v_piece * (n_pieces - 1)
+    assert tok_chunk * v_piece * 2 <= (budget or 256 << 20)
+    assert _plan(lib, n, h, v, 0, budget) == (tok_chunk, v_piece, n_chunks, n_pieces)  # memoised
 
 
 def test_forward_workspace_is_small(native):
