@@ -44,6 +44,9 @@ WORKLOADS = {
     "llama3-8b-grpo-step": dict(tokens=32768, hidden=4096, vocab=128256, dtype="bf16",
                                 temperature=1.0, ignore_frac=0.0, grpo=dict(group=64, seq=512,
                                                                             clip_eps=0.2, beta=0.04)),
+    # the logits-fed `fused_logp` scan (HBM-bound): 16384 rows of Llama-3 vocabulary, bf16 logits
+    "logits-scan": dict(tokens=16384, hidden=0, vocab=128256, dtype="bf16", temperature=1.0,
+                        ignore_frac=0.0, scan=True),
     "small": dict(tokens=4096, hidden=1024, vocab=32768, dtype="bf16", temperature=1.0,
                   ignore_frac=0.0),
 }
@@ -103,6 +106,61 @@ def cpu_baseline(torch, cfg, slice_tokens, iters=3):
     }
 
 
+def device_info(torch):
+    p = torch.cuda.get_device_properties(0)
+    khz = getattr(p, "clock_rate", 0)  # kHz where this torch build exposes it
+    info = {"name": p.name, "compute_units": p.multi_processor_count}
+    if khz:
+        info["max_sclk_mhz"] = khz / 1e3
+        info["peak_from_cu_clock_tflops"] = p.multi_processor_count * 4096 * khz * 1e3 / 1e12
+    return info
+
+
+def bench_scan(torch, args, cfg) -> int:
+    """logp from materialised logits (rlk_logp_from_logits): one pass over N x V logits."""
+    from rl_kernel_amd.ops.logp import logp_from_logits
+
+    dev = torch.device("cuda:0")
+    n, v = cfg["tokens"], cfg["vocab"]
+    dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float16
+    gen = torch.Generator(device=dev).manual_seed(1006)
+    logits = torch.empty(n, v, device=dev, dtype=dt)
+    for r0 in range(0, n, 2048):
+        logits[r0:r0 + 2048] = (torch.randn(min(2048, n - r0), v, device=dev, generator=gen) * 1.3).to(dt)
+    ids = torch.randint(0, v, (n,), device=dev, generator=gen)
+    out = torch.empty(n, device=dev, dtype=torch.float32)
+    first = logp_from_logits(logits, ids, out).clone()
+    for _ in range(args.warmup):
+        logp_from_logits(logits, ids, out)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        logp_from_logits(logits, ids, out)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    k_ms = e0.elapsed_time(e1) / args.steps
+    nbytes = float(n * v * logits.element_size() + n * 8 + n * 4)
+    result = {
+        "metric": "logp from logits tokens/sec", "value": n / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {"workload": f"logits-scan: selected-token logp from {n} x {v} {cfg['dtype']} logits",
+                   "tokens": n, "vocab": v},
+        "bitwise_repeatable": bool(torch.equal(first, out)),
+        "device": device_info(torch),
+        "roofline": {"kernel": "logp_scan_kernel", "bound": "hbm", "achieved": nbytes / (k_ms * 1e-3) / 1e9,
+                     "peak": 8000.0, "unit": "GB/s", "frac": nbytes / (k_ms * 1e-3) / 1e9 / 8000.0,
+                     "traffic": None, "algorithmic_bytes": nbytes, "launch_ms": k_ms},
+    }
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,6 +193,8 @@ def main() -> int:
     cfg = dict(WORKLOADS[args.workload])
     if args.dtype:
         cfg["dtype"] = args.dtype
+    if cfg.get("scan"):
+        return bench_scan(torch, args, cfg)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     hidden, weight, targets, grad = make_inputs(torch, cfg, dev)
@@ -264,7 +324,10 @@ def main() -> int:
         "step_frac_of_mfma_peak": step_flops / (ms * 1e-3) / 1e12 / peak,
         "step_flop_accounting": "8*N*H*V (fwd 2 + logit recompute 2 + dH 2 + dW 2)" if do_bwd
                                 else "2*N*H*V",
+        "step_tflops_no_recompute_accounting": (6.0 if do_bwd else 2.0) * n * h * v / (ms * 1e-3) / 1e12,
         "peak_extra_hbm_bytes": int(peak_extra),
+        "device": device_info(torch),
+        "seed": 1002,
         "bitwise_repeatable": bool(deterministic),
         "roofline": {
             "kernel": "linear_logp_fwd_kernel",

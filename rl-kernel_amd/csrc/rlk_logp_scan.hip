@@ -88,12 +88,44 @@ __global__ __launch_bounds__(kScanThreads) void logp_scan_kernel(
     LseState st{-INFINITY, 0.f};
     if (t < head) lse_push(st, Elem<DT>::get(x[t]));
     const u32x4* xv = reinterpret_cast<const u32x4*>(x + head);
-    for (int64_t i = t; i < nvec; i += kScanThreads) {
-        const u32x4 v = xv[i];
+    // Main scan in the log2 domain: (m2, s2) = running max of x*log2(e) and sum of 2^(x*log2e - m2).
+    // kUnroll 16-byte loads are in flight per thread; a vector first raises the max (one rescale
+    // per vector at most), then adds its terms without branches.  -inf logits add exactly 0.
+    constexpr int kUnroll = 4;
+    constexpr float kL2e = 1.4426950408889634f;
+    float m2 = -INFINITY, s2 = 0.f;
+    auto absorb = [&](const u32x4& v) {
         const E* e = reinterpret_cast<const E*>(&v);
+        float f[kPer];
+        float vmax = m2;
 #pragma unroll
-        for (int k = 0; k < kPer; ++k) lse_push(st, Elem<DT>::get(e[k]));
+        for (int k = 0; k < kPer; ++k) {
+            f[k] = Elem<DT>::get(e[k]) * kL2e;
+            vmax = fmaxf(vmax, f[k]);
+        }
+        if (vmax > m2) {
+            s2 *= __builtin_amdgcn_exp2f(m2 - vmax);  // m2 = -inf: s2 is 0 and stays 0
+            m2 = vmax;
+        }
+        const float ref = m2 == -INFINITY ? 0.f : m2;
+        float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+        for (int k = 0; k < kPer; k += 2) {
+            acc0 += __builtin_amdgcn_exp2f(f[k] - ref);
+            acc1 += __builtin_amdgcn_exp2f(f[k + 1] - ref);
+        }
+        s2 += acc0 + acc1;
+    };
+    int64_t i = t;
+    for (; i + (kUnroll - 1) * kScanThreads < nvec; i += kUnroll * kScanThreads) {
+        u32x4 v[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) v[u] = __builtin_nontemporal_load(xv + i + u * kScanThreads);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) absorb(v[u]);
     }
+    for (; i < nvec; i += kScanThreads) absorb(xv[i]);
+    if (s2 > 0.f) st = lse_merge(st, LseState{m2 * 0.6931471805599453f, s2});
     if (tail0 + t < vocab) lse_push(st, Elem<DT>::get(x[tail0 + t]));
 
     // fixed-order tree: lanes inside the wavefront, then the wavefronts through LDS
@@ -137,17 +169,39 @@ __global__ __launch_bounds__(kScanThreads) void logp_scan_bwd_kernel(
     const bool live = id >= 0 && id < vocab;
     const float c = live ? coeff[row] : 0.f;
     const float l = lse[row];
-    for (int64_t v = threadIdx.x; v < vocab; v += kScanThreads) {
-        float p = __expf(Elem<DT>::get(x[v]) - l);
+    auto value = [&](int64_t v, E xe) -> E {
+        const float p = __expf(Elem<DT>::get(xe) - l);
         float d = c * ((v == id ? 1.f : 0.f) - p);
         if (c == 0.f) d = 0.f;
-        if (DT == RLK_DTYPE_F32)
-            reinterpret_cast<float*>(g)[v] = d;
-        else if (DT == RLK_DTYPE_BF16)
-            reinterpret_cast<uint16_t*>(g)[v] = __builtin_bit_cast(uint16_t, static_cast<__bf16>(d));
+        if constexpr (DT == RLK_DTYPE_F32)
+            return d;
+        else if constexpr (DT == RLK_DTYPE_BF16)
+            return __builtin_bit_cast(uint16_t, static_cast<__bf16>(d));
         else
-            reinterpret_cast<uint16_t*>(g)[v] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
+            return __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
+    };
+    // rows of logits and gradient share their alignment when both bases are 16-byte aligned (the
+    // usual case): scalar head up to the first aligned element, 16-byte body, scalar tail
+    constexpr int kPer = 16 / sizeof(E);
+    const int t = threadIdx.x;
+    const uintptr_t ax = reinterpret_cast<uintptr_t>(x), ag = reinterpret_cast<uintptr_t>(g);
+    int64_t head = ((16 - (ax & 15)) & 15) / sizeof(E);
+    if ((ax & 15) != (ag & 15) || head > vocab) head = vocab;  // misaligned pair: all scalar
+    const int64_t nvec = (vocab - head) / kPer;
+    const int64_t tail0 = head + nvec * kPer;
+    for (int64_t v = t; v < head; v += kScanThreads) g[v] = value(v, x[v]);
+    const u32x4* xv = reinterpret_cast<const u32x4*>(x + head);
+    u32x4* gv = reinterpret_cast<u32x4*>(g + head);
+    for (int64_t i = t; i < nvec; i += kScanThreads) {
+        const u32x4 in = __builtin_nontemporal_load(xv + i);
+        u32x4 o;
+        const E* e = reinterpret_cast<const E*>(&in);
+        E* r = reinterpret_cast<E*>(&o);
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) r[k] = value(head + i * kPer + k, e[k]);
+        gv[i] = o;
     }
+    for (int64_t v = tail0 + t; v < vocab; v += kScanThreads) g[v] = value(v, x[v]);
 }
 
 }  // namespace rlk

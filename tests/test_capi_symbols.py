@@ -61,6 +61,7 @@ def test_backward_workspace_is_bounded_in_token_count(native):
     # scratch does not grow with G = 64 ... 2048: one dZ block (<= 256 MiB) + fp32 dH chunk
     assert max(sizes) <= (384 << 20) + 4096, sizes
     assert max(sizes) <= 1 << 30                # <= 1 GiB extra HBM
+    assert sizes[0] == sizes[1] == sizes[2]     # identical for G = 64, 128, 256
     need = ctypes.c_size_t(0)
     assert lib.rlk_linear_logp_bwd_workspace_bytes(131072, 2048, 151936, 1, 0, ctypes.byref(need)) == 0
     assert need.value <= 1 << 30

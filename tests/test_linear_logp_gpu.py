@@ -329,3 +329,39 @@ def test_full_size_head_properties(dev, n, h, v, dtype, temp, ign_frac, seed):
     dz[t_cpu == -100] = 0.0
     ref_dw = dz.t() @ h_cpu
     assert rel(d_w[vrows], ref_dw) < GRAD_REL
+
+
+_FRESH_PROCESS_SNIPPET = r"""
+import hashlib, sys, torch
+sys.path.insert(0, sys.argv[1])
+from rl_kernel_amd.ops import linear_logp as LL
+dev = torch.device("cuda:0")
+g = torch.Generator(device=dev).manual_seed(77)
+n, h, v = 4096, 1024, 40000
+hd = torch.randn(n, h, device=dev, generator=g).to(torch.bfloat16)
+wd = (torch.randn(v, h, device=dev, generator=g) * 0.03).to(torch.bfloat16)
+td = torch.randint(0, v, (n,), device=dev, generator=g); td[::11] = -100
+gd = torch.randn(n, device=dev, generator=g)
+logp, lse, _ = LL.fused_linear_logp_forward(hd, wd, td, temperature=0.7, ignore_index=-100)
+dh, dw, _ = LL.fused_linear_logp_backward(gd, hd, wd, td, lse, temperature=0.7, ignore_index=-100)
+m = hashlib.sha256()
+for t in (logp, lse, dh.float(), dw):
+    m.update(t.cpu().numpy().tobytes())
+print("DIGEST", m.hexdigest())
+"""
+
+
+def test_bitwise_identical_across_fresh_processes(dev):
+    """Two fresh processes on the same input give the same bits for logp, lse, dH and dW."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    digests = []
+    for _ in range(2):
+        out = subprocess.run([sys.executable, "-c", _FRESH_PROCESS_SNIPPET, root], capture_output=True,
+                             text=True, timeout=240)
+        assert out.returncode == 0, out.stderr[-2000:]
+        digests.append([l for l in out.stdout.splitlines() if l.startswith("DIGEST")][0])
+    assert digests[0] == digests[1]
