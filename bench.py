@@ -28,8 +28,8 @@ PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}  # MI355X dense MFMA, published
 # HBM bytes moved by ONE forward launch of the default workload, from two `rocprofv3 --pmc` runs of
 # this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
 # reads for the 1 GiB `--calibrate-copy` kernel (factors 2.000 and 1.000):
-# 2.000 * 24915400 KiB + 1.000 * 4608 KiB.  Other workloads report null.
-MEASURED_FWD_TRAFFIC_BYTES = {"llama3-8b-head": (2.0 * 24915400 + 4608) * 1024}
+# 2.000 * 24869400 KiB + 1.000 * 1536 KiB.  Other workloads report null.
+MEASURED_FWD_TRAFFIC_BYTES = {"llama3-8b-head": (2.0 * 24869400 + 1536) * 1024}
 
 WORKLOADS = {
     # BASELINE.json configs[1] shape; the metric is quoted on forward+backward at this shape

@@ -150,6 +150,15 @@ class _FusedLinearLogpFunction(torch.autograd.Function):
         hidden_2d = _aligned_contiguous(hidden.reshape(-1, hidden.size(-1)))
         w = _aligned_contiguous(weight)
         target_1d = target_ids.reshape(-1).to(device=hidden_2d.device, dtype=torch.long).contiguous()
+        ctx.empty = hidden_2d.size(0) == 0
+        if ctx.empty:  # no tokens: nothing to launch, gradients are zeros
+            ctx.save_for_backward(hidden_2d, w, bias if bias is not None else hidden_2d, target_1d,
+                                  hidden_2d.new_zeros(0, dtype=torch.float32))
+            ctx.has_bias = bias is not None
+            ctx.lead_shape = hidden.shape[:-1]
+            ctx.weight_dtype = weight.dtype
+            ctx.bias_dtype = bias.dtype if bias is not None else None
+            return hidden_2d.new_zeros(hidden.shape[:-1], dtype=torch.float32)
         logp, lse, err = fused_linear_logp_forward(
             hidden_2d, w, target_1d, bias, temperature=temperature, ignore_index=ignore_index)
         if check_targets and bool(err.item()):
@@ -168,6 +177,11 @@ class _FusedLinearLogpFunction(torch.autograd.Function):
         hidden_2d, w, bias_t, target_1d, lse = ctx.saved_tensors
         need_h, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[1], \
             ctx.has_bias and ctx.needs_input_grad[2]
+        if ctx.empty:
+            return (hidden_2d.new_zeros(tuple(ctx.lead_shape) + (hidden_2d.size(1),)) if need_h else None,
+                    torch.zeros_like(w, dtype=ctx.weight_dtype) if need_w else None,
+                    torch.zeros_like(bias_t, dtype=ctx.bias_dtype) if need_b else None,
+                    None, None, None, None)
         d_h, d_w, d_b = fused_linear_logp_backward(
             grad_logp, hidden_2d, w, target_1d, lse, bias_t if ctx.has_bias else None,
             temperature=ctx.temperature, ignore_index=ctx.ignore_index,

@@ -365,3 +365,15 @@ def test_bitwise_identical_across_fresh_processes(dev):
         assert out.returncode == 0, out.stderr[-2000:]
         digests.append([l for l in out.stdout.splitlines() if l.startswith("DIGEST")][0])
     assert digests[0] == digests[1]
+
+
+def test_empty_batch_returns_empty_and_zero_gradients(dev, op):
+    """No tokens (a rank whose micro-batch is empty): empty fp32 output, zero gradients."""
+    w = torch.randn(40, 16, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    b = torch.randn(40, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    h = torch.zeros(2, 0, 16, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    out = op(h, w, torch.zeros(2, 0, dtype=torch.long, device=dev), b, ignore_index=-100)
+    assert out.shape == (2, 0) and out.dtype == torch.float32
+    out.sum().backward()
+    assert h.grad.shape == h.shape
+    assert torch.count_nonzero(w.grad) == 0 and torch.count_nonzero(b.grad) == 0
