@@ -377,3 +377,52 @@ def test_empty_batch_returns_empty_and_zero_gradients(dev, op):
     out.sum().backward()
     assert h.grad.shape == h.shape
     assert torch.count_nonzero(w.grad) == 0 and torch.count_nonzero(b.grad) == 0
+
+
+def test_random_shapes_dtypes_and_dz_budgets(dev):
+    """Seeded sweep over ragged shapes (tile edges +-1, K tails, H % 8 != 0), dtypes, bias,
+    temperature, ignore-index and small dZ budgets (several token chunks x vocab pieces)."""
+    import random
+
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    rnd = random.Random(2024)
+    for case in range(32):
+        n = rnd.choice([1, 3, 64, 255, 256, 257, 300, 511, 513, 700, 1025])
+        h = rnd.choice([8, 16, 64, 72, 128, 136, 192, 256, 320, 520, 30, 7])
+        v = rnd.choice([2, 19, 255, 256, 257, 512, 777, 1024, 1500, 2304, 3001])
+        dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+        bias = rnd.random() < 0.4
+        temp = rnd.choice([1.0, 0.7, 1.3])
+        ign = rnd.random() < 0.5
+        budget = rnd.choice([0, 131072, 131072 * 2, 131072 * 6, 131072 * 12])
+        print(f"case {case}: n={n} h={h} v={v} {dtype} bias={bias} T={temp} ign={ign} "
+              f"budget={budget}", flush=True)
+        g = torch.Generator().manual_seed(case * 7919 + n + h + v)
+        hidden = torch.randn(n, h, generator=g).to(dtype)
+        weight = (torch.randn(v, h, generator=g) * h ** -0.5).to(dtype)
+        b = torch.randn(v, generator=g) if bias else None
+        tgt = torch.randint(0, v, (n,), generator=g)
+        if ign:
+            tgt[::3] = -100
+        grad = torch.randn(n, generator=g)
+        ii = -100 if ign else None
+        ref = O.linear_logp(hidden, weight, tgt, b, temperature=temp, ignore_index=ii)
+        r_dh, r_dw, r_db = O.linear_logp_backward(grad, hidden, weight, tgt, b, temperature=temp,
+                                                  ignore_index=ii)
+        hd, wd, td = hidden.to(dev), weight.to(dev), tgt.to(dev)
+        bd = None if b is None else b.to(dev)
+        logp, lse, err = LL.fused_linear_logp_forward(hd, wd, td, bd, temperature=temp,
+                                                      ignore_index=ii)
+        dh, dw, db = LL.fused_linear_logp_backward(grad.to(dev), hd, wd, td, lse, bd,
+                                                   temperature=temp, ignore_index=ii,
+                                                   dz_budget_bytes=budget)
+        atol = 1e-5 if dtype == torch.float32 else LOGP_ATOL
+        gtol = 1e-4 if dtype == torch.float32 else GRAD_REL
+        assert int(err.item()) == 0
+        assert (logp.cpu() - ref).abs().max().item() < atol
+        if ign:
+            assert torch.all(logp.cpu()[tgt == -100] == 0)
+        assert rel(dh, r_dh) < gtol and rel(dw, r_dw) < gtol
+        if bias:
+            assert rel(db, r_db) < gtol
