@@ -426,3 +426,40 @@ def test_random_shapes_dtypes_and_dz_budgets(dev):
         assert rel(dh, r_dh) < gtol and rel(dw, r_dw) < gtol
         if bias:
             assert rel(db, r_db) < gtol
+
+
+@pytest.mark.parametrize("n,h,v", [(600_000, 4096, 2048),     # N*H > 2^31 elements
+                                   (2048, 4096, 600_000)])    # V*H > 2^31 elements
+def test_element_offsets_beyond_32_bits(dev, n, h, v):
+    """Rows at the far end of a hidden / weight matrix with more than 2^31 elements: forward and
+    gradients of sampled rows against the CPU oracle (a 32-bit offset would wrap)."""
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    g = torch.Generator(device=dev).manual_seed(n + v)
+    hd = torch.empty(n, h, device=dev, dtype=torch.bfloat16)
+    for r0 in range(0, n, 65536):
+        hd[r0:r0 + 65536] = torch.randn(min(65536, n - r0), h, device=dev, generator=g).to(torch.bfloat16)
+    wd = torch.empty(v, h, device=dev, dtype=torch.bfloat16)
+    for r0 in range(0, v, 65536):
+        wd[r0:r0 + 65536] = (torch.randn(min(65536, v - r0), h, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    td = torch.randint(0, v, (n,), device=dev, generator=g)
+    td[-3:] = torch.tensor([v - 1, v - 2, 0], device=dev)      # targets at the far end of W
+    gd = torch.randn(n, device=dev, generator=g)
+    logp, lse, err = LL.fused_linear_logp_forward(hd, wd, td)
+    assert int(err.item()) == 0
+    rows = torch.tensor([0, n // 2 + 1, n - 3, n - 2, n - 1])
+    w_cpu = wd.cpu()
+    ref, ref_lse = O.linear_logp(hd[rows].cpu(), w_cpu, td[rows].cpu(), return_lse=True)
+    assert (logp[rows].cpu() - ref).abs().max().item() < LOGP_ATOL
+    d_h, d_w, _ = LL.fused_linear_logp_backward(gd, hd, wd, td, lse)
+    r_dh, _, _ = O.linear_logp_backward(gd[rows].cpu(), hd[rows].cpu(), w_cpu, td[rows].cpu())
+    assert rel(d_h[rows], r_dh) < GRAD_REL
+    # last vocab rows of dW from the definition, on the host in fp32
+    vrows = torch.tensor([0, v // 2, v - 2, v - 1])
+    h_cpu = hd.cpu().float()
+    z = h_cpu @ w_cpu[vrows].float().t()
+    t_cpu, lse_cpu, g_cpu = td.cpu(), lse.cpu(), gd.cpu()
+    dz = -(z - lse_cpu[:, None]).exp()
+    dz += (t_cpu[:, None] == vrows[None, :]).float()
+    dz *= g_cpu[:, None]
+    assert rel(d_w[vrows], dz.t() @ h_cpu) < GRAD_REL
