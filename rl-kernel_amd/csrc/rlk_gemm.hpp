@@ -34,14 +34,15 @@ typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 
 #define RLK_LDS __attribute__((address_space(3)))
 
-// Development switch for timing experiments (wrong results when non-zero): bit 0 drops the
-// global loads of the main loop, bit 1 the LDS stores, bit 2 the fragment reads, bit 3 the barrier.
-#ifndef RLK_SERP
-#define RLK_SERP 0  // 1: serpentine MFMA order (one operand changes between consecutive MFMAs)
-#endif
+// 1: the forward runs all vocab tiles of a workgroup through one pipeline (the K loop of a tile
+// fetches the head of the next); 0: every tile fills and drains its own pipeline.
 #ifndef RLK_STREAM
-#define RLK_STREAM 1  // 1: forward and dZ run all tiles of a workgroup through one pipeline
+#define RLK_STREAM 1
 #endif
+// Development switch for timing experiments (wrong results when non-zero).  Register-staged loop:
+// bit 0 drops the global loads, bit 1 the LDS stores, bit 2 the fragment reads, bit 3 the barrier,
+// bit 4 keeps unused loads alive.  Direct-to-LDS loop: bit 6 drops the global loads, bit 7 makes
+// every K step re-read the first two (always cached).  Backward kernels: bit 5 skips the epilogue.
 #ifndef RLK_ABLATE
 #define RLK_ABLATE 0
 #endif
@@ -561,7 +562,7 @@ struct TileGemmDtl {
         constexpr int wslice = last ? 0 : KKI + 1;
         static_for<0, NM>([&](auto qc) {
             constexpr int q = decltype(qc)::value;
-            constexpr int i = q / TN, j = (RLK_SERP != 0 && (i & 1)) ? TN - 1 - q % TN : q % TN;
+            constexpr int i = q / TN, j = q % TN;
             acc[i][j] = T::mfma(fa[setc][i], fb[setc][j], acc[i][j]);
             // fragment reads for the next slice: one per MFMA slot from the start of the slice, so
             // that all of them have returned when the next slice begins
