@@ -550,7 +550,7 @@ struct TileGemmDtl {
     // the last slice of the previous step.
     template <int KKI>
     __device__ static inline void slice(const IOA& la, const IOB& lb, u32x4_t (&fa)[2][TM],
-                                        u32x4_t (&fb)[2][TN], int wm, int wn, int kt, int nk,
+                                        u32x4_t (&fb)[2][TN], int wm, int wn, int kt,
                                         char* cur, char* nxt, f32x16_t (&acc)[TM][TN])
     {
         constexpr bool last = KKI == KK - 1;
@@ -656,13 +656,13 @@ struct TileGemmDtl {
             char* cur = smem + ((kt + st.phase) & 1) * kStageBytes;
             char* nxt = smem + ((kt + st.phase + 1) & 1) * kStageBytes;
             static_for<0, KK - 1>([&](auto kc) {
-                slice<decltype(kc)::value>(st.la, st.lb, st.fa, st.fb, st.wm, st.wn, kt, nk, cur,
-                                           nxt, acc);
+                slice<decltype(kc)::value>(st.la, st.lb, st.fa, st.fb, st.wm, st.wn, kt, cur, nxt,
+                                           acc);
             });
             constexpr int wait_all = vmcnt_imm(0);
             __builtin_amdgcn_s_waitcnt(wait_all);  // my loads of K step kt+1 have landed
             __syncthreads();
-            slice<KK - 1>(st.la, st.lb, st.fa, st.fb, st.wm, st.wn, kt, nk, cur, nxt, acc);
+            slice<KK - 1>(st.la, st.lb, st.fa, st.fb, st.wm, st.wn, kt, cur, nxt, acc);
         }
         st.phase = (st.phase + nk) & 1;
         st.la.base = st.la.next;

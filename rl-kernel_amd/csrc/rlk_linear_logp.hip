@@ -556,7 +556,7 @@ __global__ void linear_logp_scales_kernel(const float* grad, int n, float inv_te
     }
     red[threadIdx.x] = mx;
     __syncthreads();
-    for (int o = blockDim.x / 2; o > 0; o >>= 1) {
+    for (unsigned o = blockDim.x / 2; o > 0; o >>= 1) {
         if (threadIdx.x < o) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + o]);
         __syncthreads();
     }
