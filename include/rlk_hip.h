@@ -105,10 +105,11 @@ int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t
 
 /* Schedule the backward will use for these sizes (no counterpart in the reference, whose chunk is
  * fixed at 2^24 / V tokens, rl_engine/kernels/ops/pytorch/loss/linear_logp.py:398-400):
- * out4 = { tokens per chunk, vocab rows per piece, number of chunks, number of pieces }.  Host
- * only; touches no device. */
+ * out5 = { tokens per chunk, vocab rows per piece, number of chunks, number of pieces, parts the
+ * dH launch cuts a piece's vocab range into (1 unless there are few tokens) }.  Host only;
+ * touches no device. */
 int rlk_linear_logp_bwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype,
-                             size_t dz_budget_bytes, int64_t* out4);
+                             size_t dz_budget_bytes, int64_t* out5);
 
 int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* weight,
                         const float* bias, const int64_t* targets, const float* lse,

@@ -642,7 +642,8 @@ struct TileGemmDtl {
             st.fb[0][j] = IOB::frag(smem + IOA::kBytes, st.wn * (TN * 32) + j * 32, 0);
     }
 
-    // All K steps of the current tile into `acc`.  `next_a` / `next_b` are the operand origins of
+    // All K steps of the current tile into `acc` (callers that chain tiles need K >= 2 * BK: the
+    // loop looks two K steps ahead and knows one following tile).  `next_a` / `next_b` are the operand origins of
     // the tile that follows (same leading dimensions and row counts; pass the current origins
     // after the last tile: the extra fetches then stay inside the same tile).  On return the
     // stream stands at the start of that tile exactly as begin() leaves it.

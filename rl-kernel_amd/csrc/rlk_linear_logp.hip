@@ -139,9 +139,10 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
 
     Operand B{a.hidden + static_cast<int64_t>(tok0) * a.H, a.H, tok_valid};
     auto tile_origin = [&](int vt) { return a.weight + static_cast<int64_t>(vt) * 256 * a.H; };
-    if (!GENERAL && RLK_DTL != 0 && RLK_STREAM != 0 && a.H % BK == 0 && t0 < t1) {
+    if (!GENERAL && RLK_DTL != 0 && RLK_STREAM != 0 && a.H % BK == 0 && a.H >= 2 * BK && t0 < t1) {
         // every tile is full: one pipeline runs through all tiles of the range, the K loop of a
-        // tile already fetching the head of the next one while the softmax update runs
+        // tile already fetching the head of the next one while the softmax update runs (the
+        // pipeline looks two K steps ahead, which stays within the next tile from two steps up)
         using Dtl = TileGemmDtl<T, false, false, BK>;
         typename Dtl::Stream st;
         Dtl::begin(st, Operand{tile_origin(t0), a.H, 256}, B, a.H, smem);
@@ -388,6 +389,9 @@ struct DhArgs {
     int h_tiles;
     int first;  // 1: do not read acc
     int last;   // 1: write the 16-bit output instead of acc
+    int ksplit;           // > 1: the vocab range is cut into ksplit parts computed by separate
+    float* part;          //      workgroups, each writing its own fp32 slot [ksplit][rows][H]
+    int64_t part_stride;  //      (elements per slot); linear_logp_dh_reduce_kernel adds them up
 };
 
 template <class T, int BK>
@@ -396,15 +400,38 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
     constexpr int TM = kTM, TN = kTN;
     using Gemm = TileGemm<T, true, false, BK>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    int tt, ht;
-    xcd_tile(blockIdx.x, a.tok_tiles * a.h_tiles, a.tok_tiles, a.h_tiles, 8, tt, ht);
+    int tt, ht, ks = 0;
+    xcd_tile(blockIdx.x, a.tok_tiles * a.h_tiles * a.ksplit, a.tok_tiles, a.h_tiles * a.ksplit, 8,
+             tt, ht);
+    // K range of this workgroup: whole 64-row steps, the first (steps % ksplit) parts take one more
+    int k0 = 0, kn = a.v_valid;
+    float* acc_dst = a.acc;
+    bool first = a.first != 0, last = a.last != 0, empty_part = false;
+    if (a.ksplit > 1) {  // uniform
+        ks = ht % a.ksplit;
+        ht /= a.ksplit;
+        const int steps = (a.v_valid + BK - 1) / BK;
+        const int base = steps / a.ksplit, extra = steps % a.ksplit;
+        const int s0 = ks * base + (ks < extra ? ks : extra);
+        const int s1 = s0 + base + (ks < extra ? 1 : 0);
+        k0 = s0 * BK;
+        kn = min(a.v_valid, s1 * BK) - k0;
+        if (kn <= 0) {  // a short last piece can leave a part without K steps: it computes one
+            empty_part = true;  // step of the piece's head and discards it
+            k0 = 0;
+            kn = min(a.v_valid, BK);
+        }
+        acc_dst = a.part + static_cast<int64_t>(ks) * a.part_stride;
+        first = true;
+        last = false;
+    }
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
     const int tok0 = tt * 256, h0 = ht * 256;
 
-    Operand A{a.weight + h0, a.H, min(256, a.H - h0)};
-    Operand B{a.dz + static_cast<int64_t>(tok0) * a.ldz, a.ldz, 256};
+    Operand A{a.weight + static_cast<int64_t>(k0) * a.H + h0, a.H, min(256, a.H - h0)};
+    Operand B{a.dz + static_cast<int64_t>(tok0) * a.ldz + k0, a.ldz, 256};
     f32x16_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -412,7 +439,15 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    Gemm::run(A, B, a.v_valid, acc, smem);
+    Gemm::run(A, B, kn, acc, smem);
+    if (empty_part) {  // uniform: this part's slot must hold zeros
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    }
     if constexpr ((RLK_ABLATE & 32) != 0) { if (a.tok_valid >= 0) return; }  // dev: time without epilogue
 
     // Epilogue: all reads of the running fp32 partial are issued before the first use (clamped
@@ -432,8 +467,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
                 const int h = h0 + wm * (TM * 32) + i * 32 + 8 * q + 4 * (lane >> 5);
                 hcol[q] = h;
                 old[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-                if (!a.first)  // uniform
-                    old[q] = *reinterpret_cast<const f32x4_t*>(a.acc + trow + (h < a.H ? h : 0));
+                if (!first)  // uniform
+                    old[q] = *reinterpret_cast<const f32x4_t*>(acc_dst + trow + (h < a.H ? h : 0));
             }
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -441,18 +476,43 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
                           acc[i][j][q * 4 + 3]};
                 v += old[q];
                 if (tok_ok && hcol[q] < a.H) {  // H % 8 == 0: a quad is all-in or all-out
-                    if (a.last) {
+                    if (last) {
                         u32x2_t pk{static_cast<uint32_t>(T::from_float(v.x * oscale)) |
                                        (static_cast<uint32_t>(T::from_float(v.y * oscale)) << 16),
                                    static_cast<uint32_t>(T::from_float(v.z * oscale)) |
                                        (static_cast<uint32_t>(T::from_float(v.w * oscale)) << 16)};
                         *reinterpret_cast<u32x2_t*>(a.out + trow + hcol[q]) = pk;
                     } else {
-                        *reinterpret_cast<f32x4_t*>(a.acc + trow + hcol[q]) = v;
+                        *reinterpret_cast<f32x4_t*>(acc_dst + trow + hcol[q]) = v;
                     }
                 }
             }
         }
+    }
+}
+
+// Sum of the ksplit partial dH slots of one chunk in slot order (plus the running fp32 partial of
+// earlier vocab pieces unless `first`), written back as the running partial or, for the last
+// piece, as the 16-bit gradient.  One thread per 4 consecutive elements of a row.
+template <class T>
+__global__ void linear_logp_dh_reduce_kernel(const float* part, int ksplit, int64_t part_stride,
+                                             float* acc, uint16_t* out, const float* scales,
+                                             int64_t n4, int first, int last)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    f32x4_t v{0.f, 0.f, 0.f, 0.f};
+    if (!first) v = reinterpret_cast<const f32x4_t*>(acc)[i];
+    for (int k = 0; k < ksplit; ++k) v += reinterpret_cast<const f32x4_t*>(part + k * part_stride)[i];
+    if (last) {
+        const float oscale = scales[1];
+        u32x2_t pk{static_cast<uint32_t>(T::from_float(v.x * oscale)) |
+                       (static_cast<uint32_t>(T::from_float(v.y * oscale)) << 16),
+                   static_cast<uint32_t>(T::from_float(v.z * oscale)) |
+                       (static_cast<uint32_t>(T::from_float(v.w * oscale)) << 16)};
+        reinterpret_cast<u32x2_t*>(out)[i] = pk;
+    } else {
+        reinterpret_cast<f32x4_t*>(acc)[i] = v;
     }
 }
 
@@ -655,9 +715,11 @@ struct BwdPlan {
     int v_piece;     // vocab rows per piece (multiple of 256)
     int n_chunks;
     int n_pieces;
+    int ksplit;      // dH launch: parts of the piece's vocab range computed side by side
     size_t dz_bytes;
     size_t acc_bytes;
-    size_t scales_off, dz_off, acc_off, total;
+    size_t part_bytes;
+    size_t scales_off, dz_off, acc_off, part_off, total;
 };
 
 // Cost of the three launches of one dZ block of ct x pt tiles, in K steps of one CU: a launch of
@@ -736,7 +798,19 @@ BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
     p.scales_off = 0;
     p.dz_off = 256;
     p.acc_off = p.dz_off + align_up(p.dz_bytes, 256);
-    p.total = p.acc_off + align_up(p.acc_bytes, 256);
+    // Few tokens: the dH launch has fewer tiles than the chip has CUs but a long vocab range, so
+    // the range is cut into parts that run side by side and are added up in a fixed order.
+    p.ksplit = 1;
+    const int64_t dh_tiles = best_ct * ht;
+    if (dh_tiles <= 128 && best_pt >= 32) {
+        int64_t lim = 256 / dh_tiles;
+        if (lim > best_pt / 16) lim = best_pt / 16;
+        if (lim > 8) lim = 8;
+        while (p.ksplit * 2 <= lim) p.ksplit *= 2;
+    }
+    p.part_bytes = p.ksplit > 1 ? static_cast<size_t>(p.ksplit) * p.tok_chunk * H * 4 : 0;
+    p.part_off = p.acc_off + align_up(p.acc_bytes, 256);
+    p.total = p.part_off + align_up(p.part_bytes, 256);
     memo = Key{N, V, H, budget, p};
     return p;
 }
@@ -898,17 +972,18 @@ int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t
 }
 
 int rlk_linear_logp_bwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype, size_t dz_budget_bytes,
-                             int64_t* out4)
+                             int64_t* out5)
 {
     (void)dtype;
-    if (!out4 || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad plan query");
+    if (!out5 || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad plan query");
     if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
     if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
     const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
-    out4[0] = p.tok_chunk;
-    out4[1] = p.v_piece;
-    out4[2] = p.n_chunks;
-    out4[3] = p.n_pieces;
+    out5[0] = p.tok_chunk;
+    out5[1] = p.v_piece;
+    out5[2] = p.n_chunks;
+    out5[3] = p.n_pieces;
+    out5[4] = p.ksplit;
     return 0;
 }
 
@@ -1010,6 +1085,9 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
             h.h_tiles = h_tiles;
             h.first = pi == 0;
             h.last = last_piece;
+            h.ksplit = p.ksplit;
+            h.part = p.ksplit > 1 ? reinterpret_cast<float*>(ws + p.part_off) : nullptr;
+            h.part_stride = static_cast<int64_t>(p.tok_chunk) * H;
 
             DwArgs d;
             d.dz = dz;
@@ -1043,9 +1121,18 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                                        dim3(tok_tiles * gen_tiles), dim3(kThreads), GZb::kSmemBytes,
                                        stream, z);
                 }
-                if (d_hidden)
-                    hipLaunchKernelGGL((linear_logp_dh_kernel<Bf16, kBK>), dim3(tok_tiles * h_tiles),
-                                       dim3(kThreads), GHb::kSmemBytes, stream, h);
+                if (d_hidden) {
+                    hipLaunchKernelGGL((linear_logp_dh_kernel<Bf16, kBK>),
+                                       dim3(tok_tiles * h_tiles * p.ksplit), dim3(kThreads),
+                                       GHb::kSmemBytes, stream, h);
+                    if (p.ksplit > 1) {
+                        const int64_t n4 = static_cast<int64_t>(tok_valid) * H / 4;
+                        hipLaunchKernelGGL((linear_logp_dh_reduce_kernel<Bf16>),
+                                           dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0,
+                                           stream, h.part, p.ksplit, h.part_stride, h.acc, h.out,
+                                           scales, n4, h.first, h.last);
+                    }
+                }
                 if (d_weight)
                     hipLaunchKernelGGL((linear_logp_dw_kernel<Bf16, kBK>), dim3(v_tiles * h_tiles),
                                        dim3(kThreads), GWb::kSmemBytes, stream, d);
@@ -1064,9 +1151,18 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                                        dim3(tok_tiles * gen_tiles), dim3(kThreads), GZb::kSmemBytes,
                                        stream, z);
                 }
-                if (d_hidden)
-                    hipLaunchKernelGGL((linear_logp_dh_kernel<F16, kBK>), dim3(tok_tiles * h_tiles),
-                                       dim3(kThreads), GHb::kSmemBytes, stream, h);
+                if (d_hidden) {
+                    hipLaunchKernelGGL((linear_logp_dh_kernel<F16, kBK>),
+                                       dim3(tok_tiles * h_tiles * p.ksplit), dim3(kThreads),
+                                       GHb::kSmemBytes, stream, h);
+                    if (p.ksplit > 1) {
+                        const int64_t n4 = static_cast<int64_t>(tok_valid) * H / 4;
+                        hipLaunchKernelGGL((linear_logp_dh_reduce_kernel<F16>),
+                                           dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0,
+                                           stream, h.part, p.ksplit, h.part_stride, h.acc, h.out,
+                                           scales, n4, h.first, h.last);
+                    }
+                }
                 if (d_weight)
                     hipLaunchKernelGGL((linear_logp_dw_kernel<F16, kBK>), dim3(v_tiles * h_tiles),
                                        dim3(kThreads), GWb::kSmemBytes, stream, d);

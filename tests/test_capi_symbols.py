@@ -46,7 +46,7 @@ def test_binding_covers_every_declared_symbol(native):
 
 
 def _plan(lib, n, h, v, dtype=0, budget=0):
-    out = (ctypes.c_int64 * 4)()
+    out = (ctypes.c_int64 * 5)()
     assert lib.rlk_linear_logp_bwd_plan(n, h, v, dtype, budget, out) == 0
     return tuple(out)
 
@@ -72,12 +72,13 @@ def test_backward_workspace_is_bounded_in_token_count(native):
 @pytest.mark.parametrize("budget", [0, 64 << 20, 1 << 30])
 def test_backward_plan_covers_the_problem_within_budget(native, n, h, v, budget):
     lib = native.load()
-    tok_chunk, v_piece, n_chunks, n_pieces = _plan(lib, n, h, v, 0, budget)
+    tok_chunk, v_piece, n_chunks, n_pieces, dh_parts = _plan(lib, n, h, v, 0, budget)
+    assert dh_parts in (1, 2, 4, 8)
     assert tok_chunk % 256 == 0 and v_piece % 256 == 0 and tok_chunk > 0 and v_piece > 0
     assert tok_chunk * n_chunks >= n > tok_chunk * (n_chunks - 1)
     assert v_piece * n_pieces >= v > v_piece * (n_pieces - 1)
     assert tok_chunk * v_piece * 2 <= (budget or 256 << 20)
-    assert _plan(lib, n, h, v, 0, budget) == (tok_chunk, v_piece, n_chunks, n_pieces)  # memoised
+    assert _plan(lib, n, h, v, 0, budget) == (tok_chunk, v_piece, n_chunks, n_pieces, dh_parts)  # memoised
 
 
 def test_forward_workspace_is_small(native):
@@ -114,3 +115,12 @@ def test_missing_library_fails_loudly(native, monkeypatch, tmp_path):
     with pytest.raises(native.NativeLibraryError, match="no CPU or PyTorch fallback"):
         native.load()
     assert native.available() is False
+
+
+def test_backward_plan_splits_dh_only_for_few_tokens(native):
+    lib = native.load()
+    assert _plan(lib, 32768, 4096, 128256)[4] == 1
+    assert _plan(lib, 4096, 4096, 128256)[4] == 1
+    assert _plan(lib, 1024, 4096, 128256)[4] == 4      # 64 dH tiles on 256 CUs
+    assert _plan(lib, 2048, 4096, 128256)[4] == 2
+    assert _plan(lib, 300, 64, 40000)[4] > 1

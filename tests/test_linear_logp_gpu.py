@@ -57,6 +57,9 @@ CASES = [
     ((300,), 136, 1500, torch.bfloat16, True, 1.0, 0.0),    # H not a multiple of the K step
     ((1000,), 128, 2304, torch.bfloat16, False, 1.0, 0.01),  # V a multiple of 256: fast path only
     ((64,), 2048, 5120, torch.float16, False, 1.0, 0.0),
+    ((300,), 64, 40000, torch.bfloat16, False, 1.0, 0.0),    # one K step, several tiles per workgroup
+    ((300,), 128, 40000, torch.float16, False, 0.7, 0.1),    # two K steps, several tiles per workgroup
+    ((700,), 192, 70000, torch.bfloat16, False, 1.0, 0.0),
 ]
 
 
@@ -463,3 +466,34 @@ def test_element_offsets_beyond_32_bits(dev, n, h, v):
     dz += (t_cpu[:, None] == vrows[None, :]).float()
     dz *= g_cpu[:, None]
     assert rel(d_w[vrows], dz.t() @ h_cpu) < GRAD_REL
+
+
+@pytest.mark.parametrize("n,h,v,dtype,budget", [
+    (300, 64, 40000, torch.bfloat16, 0),           # one piece, dH range cut into parts
+    (513, 128, 70001, torch.float16, 16 << 20),    # several pieces, ragged last piece and K tail
+    (1024, 256, 32868, torch.bfloat16, 32 << 20),  # 100-row last piece: two of four parts stay empty
+])
+def test_few_tokens_long_vocab_split_dh(dev, n, h, v, dtype, budget):
+    """Few tokens against a long vocabulary: the dH launch cuts each vocab piece into parts that
+    run side by side (checked through the plan query) and must still match the oracle."""
+    import ctypes
+
+    from rl_kernel_amd import _native
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    plan = (ctypes.c_int64 * 5)()
+    assert _native.load().rlk_linear_logp_bwd_plan(n, h, v, 0, budget, plan) == 0
+    assert plan[4] > 1, list(plan)
+    hidden, weight, _, tgt, grad = make(31, (n,), h, v, dtype, False, 0.1)
+    ref = O.linear_logp(hidden, weight, tgt, ignore_index=-100)
+    r_dh, r_dw, _ = O.linear_logp_backward(grad, hidden, weight, tgt, ignore_index=-100)
+    hd, wd, td = hidden.to(dev), weight.to(dev), tgt.to(dev)
+    logp, lse, _ = LL.fused_linear_logp_forward(hd, wd, td, ignore_index=-100)
+    dh, dw, _ = LL.fused_linear_logp_backward(grad.to(dev), hd, wd, td, lse, ignore_index=-100,
+                                              dz_budget_bytes=budget)
+    dh2, dw2, _ = LL.fused_linear_logp_backward(grad.to(dev), hd, wd, td, lse, ignore_index=-100,
+                                                dz_budget_bytes=budget)
+    assert (logp.cpu() - ref).abs().max().item() < LOGP_ATOL
+    assert rel(dh, r_dh) < GRAD_REL and rel(dw, r_dw) < GRAD_REL
+    assert torch.equal(dh, dh2) and torch.equal(dw, dw2)
+    assert torch.all(dh.float().cpu()[tgt == -100] == 0)
