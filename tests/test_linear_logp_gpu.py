@@ -390,15 +390,15 @@ def test_random_shapes_dtypes_and_dz_budgets(dev):
     from rl_kernel_amd.ops import linear_logp as LL
 
     rnd = random.Random(2024)
-    for case in range(32):
+    for case in range(40):
         n = rnd.choice([1, 3, 64, 255, 256, 257, 300, 511, 513, 700, 1025])
         h = rnd.choice([8, 16, 64, 72, 128, 136, 192, 256, 320, 520, 30, 7])
-        v = rnd.choice([2, 19, 255, 256, 257, 512, 777, 1024, 1500, 2304, 3001])
+        v = rnd.choice([2, 19, 255, 256, 257, 512, 777, 1024, 1500, 2304, 3001, 20000, 40000])
         dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
         bias = rnd.random() < 0.4
         temp = rnd.choice([1.0, 0.7, 1.3])
         ign = rnd.random() < 0.5
-        budget = rnd.choice([0, 131072, 131072 * 2, 131072 * 6, 131072 * 12])
+        budget = rnd.choice([0, 131072, 131072 * 2, 131072 * 6, 131072 * 12, 8 << 20])
         print(f"case {case}: n={n} h={h} v={v} {dtype} bias={bias} T={temp} ign={ign} "
               f"budget={budget}", flush=True)
         g = torch.Generator().manual_seed(case * 7919 + n + h + v)
