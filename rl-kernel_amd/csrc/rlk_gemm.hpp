@@ -90,6 +90,13 @@ struct Bf16 {
     {
         return __builtin_bit_cast(float, static_cast<uint32_t>(x) << 16);
     }
+    // two values rounded and packed by one conversion instruction (lo in bits 0..15)
+    __device__ static inline uint32_t pack2(float lo, float hi)
+    {
+        typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+        typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+    }
 };
 
 struct F16 {
@@ -107,6 +114,12 @@ struct F16 {
     __device__ static inline float to_float(uint16_t x)
     {
         return static_cast<float>(__builtin_bit_cast(_Float16, x));
+    }
+    __device__ static inline uint32_t pack2(float lo, float hi)
+    {
+        typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+        typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, f16x2_t));
     }
 };
 

@@ -334,29 +334,43 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
                              : -1;
         // the 16-bit tile is staged in LDS as [token][vocab] rows so that it leaves in full lines
         char* srow = smem + tl * kDzPitch + (wm * (TM * 32) + 4 * (lane >> 5)) * 2;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t o[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int r = q * 4 + c;
-                    float z = acc[i][j][r];
-                    float p;
-                    if (GENERAL) {
-                        const int v = vw + i * 32 + acc_row(r, lane);
-                        if (a.bias != nullptr) z += a.bias[v < a.v_valid ? v : a.v_valid - 1];
-                        p = v < a.v_valid ? __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2)) : 0.f;
-                    } else {
-                        p = __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2));
-                    }
-                    const float hit = (etgt == i * 16 + r) ? gs : 0.f;
-                    o[c] = T::from_float(fmaf(-gs, p, hit));
-                }
-                u32x2_t pk{o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
-                *reinterpret_cast<u32x2_t*>(srow + (i * 32 + 8 * q) * 2) = pk;
+        auto prob = [&](int i, int r) -> float {
+            float z = acc[i][j][r];
+            if (GENERAL) {
+                const int v = vw + i * 32 + acc_row(r, lane);
+                if (a.bias != nullptr) z += a.bias[v < a.v_valid ? v : a.v_valid - 1];
+                return v < a.v_valid ? __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2)) : 0.f;
             }
+            return __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2));
+        };
+        // the one-hot term is added only when some lane of the wavefront owns its target row in
+        // this slab; values are rounded and packed two at a time
+        if (__builtin_amdgcn_ballot_w64(etgt >= 0) != 0) {  // uniform
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float d[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int r = q * 4 + c;
+                        const float hit = (etgt == i * 16 + r) ? gs : 0.f;
+                        d[c] = fmaf(-gs, prob(i, r), hit);
+                    }
+                    *reinterpret_cast<u32x2_t*>(srow + (i * 32 + 8 * q) * 2) =
+                        u32x2_t{T::pack2(d[0], d[1]), T::pack2(d[2], d[3])};
+                }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float d0 = -gs * prob(i, q * 4 + 0), d1 = -gs * prob(i, q * 4 + 1);
+                    const float d2 = -gs * prob(i, q * 4 + 2), d3 = -gs * prob(i, q * 4 + 3);
+                    *reinterpret_cast<u32x2_t*>(srow + (i * 32 + 8 * q) * 2) =
+                        u32x2_t{T::pack2(d0, d1), T::pack2(d2, d3)};
+                }
+        }
     }
     __syncthreads();
     // copy-out: a half wavefront moves one 512-byte row (4 full lines), 16 bytes per lane
