@@ -373,16 +373,18 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
         }
     }
     __syncthreads();
-    // copy-out: a half wavefront moves one 512-byte row (4 full lines), 16 bytes per lane
+    // copy-out: a half wavefront moves one 512-byte row (4 full lines) as two runs of 32 x 8
+    // consecutive bytes (consecutive lanes read consecutive LDS banks)
     uint16_t* dtile = a.dz + static_cast<int64_t>(tok0) * a.ldz + v0;
 #pragma unroll 4
     for (int it = 0; it < 256 / (2 * (kThreads / 64)); ++it) {
         const int row = it * (2 * (kThreads / 64)) + 2 * wave + (lane >> 5);
-        const char* src = smem + row * kDzPitch + (lane & 31) * 16;  // 8-byte aligned (pitch)
+        const char* src = smem + row * kDzPitch + (lane & 31) * 8;  // 8-byte aligned (pitch)
         const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(src);
-        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(src + 8);
-        *reinterpret_cast<u32x4_t*>(dtile + static_cast<int64_t>(row) * a.ldz + (lane & 31) * 8) =
-            u32x4_t{lo.x, lo.y, hi.x, hi.y};
+        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(src + 256);
+        uint16_t* dst = dtile + static_cast<int64_t>(row) * a.ldz + (lane & 31) * 4;
+        *reinterpret_cast<u32x2_t*>(dst) = lo;
+        *reinterpret_cast<u32x2_t*>(dst + 128) = hi;
     }
 }
 
@@ -491,10 +493,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
                 v += old[q];
                 if (tok_ok && hcol[q] < a.H) {  // H % 8 == 0: a quad is all-in or all-out
                     if (last) {
-                        u32x2_t pk{static_cast<uint32_t>(T::from_float(v.x * oscale)) |
-                                       (static_cast<uint32_t>(T::from_float(v.y * oscale)) << 16),
-                                   static_cast<uint32_t>(T::from_float(v.z * oscale)) |
-                                       (static_cast<uint32_t>(T::from_float(v.w * oscale)) << 16)};
+                        u32x2_t pk{T::pack2(v.x * oscale, v.y * oscale), T::pack2(v.z * oscale, v.w * oscale)};
                         *reinterpret_cast<u32x2_t*>(a.out + trow + hcol[q]) = pk;
                     } else {
                         *reinterpret_cast<f32x4_t*>(acc_dst + trow + hcol[q]) = v;
@@ -520,10 +519,7 @@ __global__ void linear_logp_dh_reduce_kernel(const float* part, int ksplit, int6
     for (int k = 0; k < ksplit; ++k) v += reinterpret_cast<const f32x4_t*>(part + k * part_stride)[i];
     if (last) {
         const float oscale = scales[1];
-        u32x2_t pk{static_cast<uint32_t>(T::from_float(v.x * oscale)) |
-                       (static_cast<uint32_t>(T::from_float(v.y * oscale)) << 16),
-                   static_cast<uint32_t>(T::from_float(v.z * oscale)) |
-                       (static_cast<uint32_t>(T::from_float(v.w * oscale)) << 16)};
+        u32x2_t pk{T::pack2(v.x * oscale, v.y * oscale), T::pack2(v.z * oscale, v.w * oscale)};
         reinterpret_cast<u32x2_t*>(out)[i] = pk;
     } else {
         reinterpret_cast<f32x4_t*>(acc)[i] = v;
