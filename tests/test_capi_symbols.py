@@ -124,3 +124,19 @@ def test_backward_plan_splits_dh_only_for_few_tokens(native):
     assert _plan(lib, 1024, 4096, 128256)[4] == 4      # 64 dH tiles on 256 CUs
     assert _plan(lib, 2048, 4096, 128256)[4] == 2
     assert _plan(lib, 300, 64, 40000)[4] > 1
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/rlk_hip.h must compile as C (no C++ or torch types in the boundary)."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("gcc not available")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "rlk_hip.h"\nint main(void) { return rlk_version() < 0; }\n')
+    res = subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-fsyntax-only",
+                          "-I", os.path.join(ROOT, "include"), str(src)],
+                         capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
