@@ -172,6 +172,8 @@ def main() -> int:
     ap.add_argument("--mode", default="fwd+bwd", choices=["fwd+bwd", "fwd"])
     ap.add_argument("--dtype", default=None, choices=["bf16", "f16"],
                     help="override the workload's 16-bit input type")
+    ap.add_argument("--no-library-gemm", action="store_true",
+                    help="skip the vendor-GEMM comparison figure")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known HBM traffic) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
@@ -342,6 +344,26 @@ def main() -> int:
             "flops_per_launch": fwd_flops,
         },
     }
+    if not args.no_library_gemm:
+        # vendor GEMM (torch.matmul -> hipBLASLt) on the same box at the same H, for scale only:
+        # hidden [N, H] x W[:16384]^T -> [N, 16384] in the input dtype
+        try:
+            wv = weight[: min(v, 16384)]
+            torch.matmul(hidden, wv.t())
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                torch.matmul(hidden, wv.t())
+            e1.record()
+            torch.cuda.synchronize()
+            lib_ms = e0.elapsed_time(e1) / 5
+            result["library_gemm"] = {
+                "what": f"torch.matmul [{n},{h}] x [{h},{wv.shape[0]}] {cfg['dtype']} (writes the logits it computes)",
+                "tflops": 2.0 * n * h * wv.shape[0] / (lib_ms * 1e-3) / 1e12, "ms": lib_ms}
+        except Exception as exc:  # the comparison is optional
+            result["library_gemm"] = {"error": str(exc)[:200]}
     if grpo:
         epi_ms = sum(a.elapsed_time(b) for a, b in epi_ev) / len(epi_ev)
         epi_bytes = n * (4 + 4 + 4 + 1 + 4 + 4)  # cur, old, ref, mask in; d_cur, d_kl out
