@@ -84,6 +84,23 @@ int rlk_linear_logp_fwd(const void* hidden, const void* weight, const float* bia
                         int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
                         int32_t* err_flag, rlk_stream_t stream);
 
+/* Forward for callers that cannot allocate or pass a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, kernels and bits as rlk_linear_logp_fwd, but the per-split partial softmax
+ * states live in a file-scope device array of RLK_STATIC_SCRATCH_BYTES inside the library (one
+ * copy per GPU, held until the process ends) instead of `workspace`; the call allocates and frees
+ * nothing.  Sizes whose partials (rlk_linear_logp_fwd_workspace_bytes) exceed that array are
+ * rejected with RLK_ERR_ARG.  All calls on one GPU share the array: calls that overlap in time on
+ * the same GPU (different streams or threads) race; serialise them.  Nothing in the array needs to
+ * start at zero (every slot that is read was written by the same call). */
+#define RLK_STATIC_SCRATCH_BYTES (8u << 20)
+
+int rlk_linear_logp_fwd_static(const void* hidden, const void* weight, const float* bias,
+                               const int64_t* targets, float* logp, float* lse, int64_t N,
+                               int32_t H, int64_t V, int64_t vocab_start, int32_t dtype,
+                               float temperature, int64_t ignore_index, int32_t use_ignore,
+                               int32_t strict_targets, int32_t* err_flag, rlk_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------ *
  * Fused linear -> log-prob, backward.
  *

@@ -7,6 +7,7 @@
 // forward and in the dZ recompute M = vocab and N = token, so one lane owns whole token columns
 // and the softmax reduction over vocab is a plain in-register loop with no cross-lane traffic.
 #include "rlk_common.hpp"
+#include <mutex>
 #include <vector>
 
 #include "rlk_gemm.hpp"
@@ -857,6 +858,47 @@ bool use_mfma(const void* hidden, const void* weight, int32_t H, int dtype)
            (reinterpret_cast<uintptr_t>(hidden) & 15) == 0 && (reinterpret_cast<uintptr_t>(weight) & 15) == 0;
 }
 
+int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const int64_t* targets,
+                float* logp, float* lse, void* workspace, size_t workspace_bytes, int64_t N,
+                int32_t H, int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
+                int32_t* err_flag, hipStream_t stream);
+
+}  // namespace
+
+// Scratch of rlk_linear_logp_fwd_static: the forward's per-split partial softmax states live in
+// this file-scope device array instead of a caller workspace, so that entry point allocates
+// nothing.  Every GPU the library runs on holds its own copy until the process ends.  In host code
+// the array's name is only a handle; the device address is looked up once per device below and
+// that pointer is what the kernels receive.
+static __device__ __align__(256) unsigned char scratch[RLK_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (resolved on the first call per device).
+int static_scratch_ptr(void** out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return rlk_fail(RLK_ERR_UNSUPPORTED, "device index too large");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return rlk_fail(RLK_ERR_LAUNCH, e != hipSuccess ? hipGetErrorString(e)
+                                                            : "static scratch has no device address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -879,6 +921,42 @@ int rlk_linear_logp_fwd(const void* hidden, const void* weight, const float* bia
                         int64_t vocab_start, int32_t dtype, float temperature,
                         int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
                         int32_t* err_flag, hipStream_t stream)
+{
+    return fwd_enqueue(hidden, weight, bias, targets, logp, lse, workspace, workspace_bytes, N, H, V,
+                       vocab_start, dtype, temperature, ignore_index, use_ignore, strict_targets,
+                       err_flag, stream);
+}
+
+int rlk_linear_logp_fwd_static(const void* hidden, const void* weight, const float* bias,
+                               const int64_t* targets, float* logp, float* lse, int64_t N,
+                               int32_t H, int64_t V, int64_t vocab_start, int32_t dtype,
+                               float temperature, int64_t ignore_index, int32_t use_ignore,
+                               int32_t strict_targets, int32_t* err_flag, hipStream_t stream)
+{
+    if (int rc = check_common(N, H, V, dtype)) return rc;
+    size_t need = 0;
+    if (int rc = rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &need)) return rc;
+    if (need > static_cast<size_t>(RLK_STATIC_SCRATCH_BYTES))
+        return rlk_fail(RLK_ERR_ARG,
+                        "rlk_linear_logp_fwd_static: the split partials of this N exceed the "
+                        "library's static scratch (RLK_STATIC_SCRATCH_BYTES); use "
+                        "rlk_linear_logp_fwd with a caller workspace");
+    void* ws = nullptr;
+    if (int rc = static_scratch_ptr(&ws)) return rc;
+    return fwd_enqueue(hidden, weight, bias, targets, logp, lse, ws, RLK_STATIC_SCRATCH_BYTES, N, H,
+                       V, vocab_start, dtype, temperature, ignore_index, use_ignore,
+                       strict_targets, err_flag, stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const int64_t* targets,
+                float* logp, float* lse, void* workspace, size_t workspace_bytes, int64_t N,
+                int32_t H, int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
+                int32_t* err_flag, hipStream_t stream)
 {
     if (int rc = check_common(N, H, V, dtype)) return rc;
     if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
@@ -960,6 +1038,10 @@ int rlk_linear_logp_fwd(const void* hidden, const void* weight, const float* bia
     hipLaunchKernelGGL(linear_logp_combine_kernel, dim3((a.N + 255) / 256), dim3(256), 0, stream, c);
     return check_launch("linear_logp_combine_kernel launch failed");
 }
+
+}  // namespace
+
+extern "C" {
 
 int rlk_selftest_transpose_read(int32_t* out, hipStream_t stream)
 {

@@ -1,0 +1,94 @@
+"""rlk_linear_logp_fwd_static (the forward entry point that allocates nothing: its split partials
+live in a device array inside the library) must return the bits of rlk_linear_logp_fwd, also on a
+second call with a smaller input that reuses the same array."""
+import ctypes
+
+import pytest
+
+torch = pytest.importorskip("torch")
+
+pytestmark = pytest.mark.gpu
+
+
+def _call_pair(lib, n, h, v, dtype, seed, temperature, with_ignore, with_bias):
+    from rl_kernel_amd import _native
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(seed)
+    hidden = torch.randn(n, h, generator=g).to(dtype).to(dev)
+    weight = (torch.randn(v, h, generator=g) * 0.05).to(dtype).to(dev)
+    targets = torch.randint(0, v, (n,), generator=g)
+    if with_ignore:
+        targets[::7] = -100
+    targets = targets.to(dev)
+    bias = (torch.randn(v, generator=g) * 0.1).to(dev) if with_bias else None
+    dt = {torch.bfloat16: _native.DTYPE_BF16, torch.float16: _native.DTYPE_F16}[dtype]
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    need = ctypes.c_size_t(0)
+    assert lib.rlk_linear_logp_fwd_workspace_bytes(n, h, v, dt, ctypes.byref(need)) == 0
+    ws = torch.empty(max(need.value, 16), device=dev, dtype=torch.uint8)
+    outs = []
+    for static in (False, True):
+        # outputs pre-filled with a sentinel so that an unwritten slot cannot pass by accident
+        logp = torch.full((n,), 123.0, device=dev)
+        lse = torch.full((n,), -77.0, device=dev)
+        err = torch.zeros(1, device=dev, dtype=torch.int32)
+        common = (n, h, v, 0, dt, float(temperature), -100, int(with_ignore), 1, err.data_ptr(),
+                  stream)
+        bias_p = None if bias is None else bias.data_ptr()
+        if static:
+            before = torch.cuda.memory_allocated(dev)
+            rc = lib.rlk_linear_logp_fwd_static(hidden.data_ptr(), weight.data_ptr(), bias_p,
+                                                targets.data_ptr(), logp.data_ptr(),
+                                                lse.data_ptr(), *common)
+            assert torch.cuda.memory_allocated(dev) == before
+        else:
+            rc = lib.rlk_linear_logp_fwd(hidden.data_ptr(), weight.data_ptr(), bias_p,
+                                         targets.data_ptr(), logp.data_ptr(), lse.data_ptr(),
+                                         ws.data_ptr(), ws.numel(), *common)
+        assert rc == 0, lib.rlk_last_error()
+        torch.cuda.synchronize()
+        assert int(err.item()) == 0
+        outs.append((logp.cpu(), lse.cpu()))
+    return outs, (hidden, weight, targets, bias)
+
+
+def test_static_scratch_forward_matches_the_workspace_forward_twice():
+    from oracle import oracle as O
+    from rl_kernel_amd import _native
+
+    lib = _native.load()
+    # first call: several vocab splits and a ragged last token block / vocab tile; second call:
+    # a smaller input, which must not see anything the first one left in the array
+    cases = [(1500, 256, 9000, torch.bfloat16, 5, 0.7, True, False),
+             (300, 128, 1000, torch.float16, 6, 1.0, False, True)]
+    for n, h, v, dtype, seed, temp, ign, with_bias in cases:
+        (ref, got), (hidden, weight, targets, bias) = _call_pair(lib, n, h, v, dtype, seed, temp,
+                                                                 ign, with_bias)
+        assert torch.equal(ref[0], got[0]) and torch.equal(ref[1], got[1])  # same kernels, same bits
+        want = O.linear_logp(hidden.cpu(), weight.cpu(), targets.cpu(),
+                             None if bias is None else bias.cpu(), temperature=temp,
+                             ignore_index=-100 if ign else None)
+        assert (got[0] - want).abs().max().item() < 1e-3   # bf16 / f16 inputs, fp32 accumulate
+        if ign:
+            assert torch.equal(got[0][targets.cpu() == -100], torch.zeros((n + 6) // 7))
+
+
+def test_static_scratch_forward_rejects_sizes_beyond_its_array():
+    from rl_kernel_amd import _native
+
+    lib = _native.load()
+    n, h, v = 1 << 22, 4096, 128256   # partials of 4 M tokens do not fit 8 MiB
+    need = ctypes.c_size_t(0)
+    assert lib.rlk_linear_logp_fwd_workspace_bytes(n, h, v, 0, ctypes.byref(need)) == 0
+    assert need.value > 8 << 20
+    dev = torch.device("cuda:0")
+    dummy = torch.zeros(64, device=dev)
+    err = torch.zeros(1, device=dev, dtype=torch.int32)
+    rc = lib.rlk_linear_logp_fwd_static(dummy.data_ptr(), dummy.data_ptr(), None, dummy.data_ptr(),
+                                        dummy.data_ptr(), dummy.data_ptr(), n, h, v, 0, 0, 1.0, 0,
+                                        0, 1, err.data_ptr(),
+                                        torch.cuda.current_stream(dev).cuda_stream)
+    assert rc == -1   # RLK_ERR_ARG, nothing enqueued
+    assert b"static scratch" in lib.rlk_last_error()
