@@ -39,14 +39,6 @@ typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 #ifndef RLK_STREAM
 #define RLK_STREAM 1
 #endif
-// Development switch for timing experiments (wrong results when non-zero).  Register-staged loop:
-// bit 0 drops the global loads, bit 1 the LDS stores, bit 2 the fragment reads, bit 3 the barrier,
-// bit 4 keeps unused loads alive.  Direct-to-LDS loop: bit 6 drops the global loads, bit 7 makes
-// every K step re-read the first two (always cached).  Backward kernels: bit 5 skips the epilogue.
-#ifndef RLK_ABLATE
-#define RLK_ABLATE 0
-#endif
-
 // Main-loop variant: 1 = global memory is copied straight into LDS (no staging registers),
 // 0 = global -> registers -> LDS.  K steps that are not a whole BK always take the second.
 #ifndef RLK_DTL
@@ -185,13 +177,13 @@ struct TileIO {
         const int t = threadIdx.x;
         const int chunk = t % G::kChunksPerLine;
         const int line0 = t / G::kChunksPerLine;
-        const uint32_t adv = static_cast<uint32_t>(kt) * step;
+        const size_t adv = static_cast<size_t>(kt) * step;  // 64-bit: K * ld can pass 4 GiB
 #pragma unroll
         for (int p = 0; p < G::kPasses; ++p) {
             if (CHECKED) {
                 const int k = kt * BK + (KMAJOR ? p * G::kLinesPerPass + line0 : chunk * 8);
                 const bool live = k < K;
-                const uint32_t o = live ? off[p] + adv : off[p];
+                const size_t o = live ? off[p] + adv : off[p];
                 u32x4_t v = *reinterpret_cast<const u32x4_t*>(base + o);
                 if (!live) v = u32x4_t{0u, 0u, 0u, 0u};
                 reg[p] = v;
@@ -214,8 +206,8 @@ struct TileIO {
     template <bool CHECKED>
     __device__ inline void load_one(int kt, int K, u32x4_t (&reg)[G::kPasses], int p) const
     {
-        const uint32_t adv = static_cast<uint32_t>(kt) * step;
-        uint32_t o = off[p] + adv;
+        const size_t adv = static_cast<size_t>(kt) * step;  // 64-bit: K * ld can pass 4 GiB
+        size_t o = off[p] + adv;
         if (CHECKED) o = live(kt, K, p) ? o : off[p];
         reg[p] = *reinterpret_cast<const u32x4_t*>(base + o);
     }
@@ -338,8 +330,7 @@ struct TileGemm {
             // order the next slice's MFMAs (i-major) first need them: A0, B0..B(TN-1), A1..A(TM-1)
             static_for<q * NR / NM, (q + 1) * NR / NM>([&](auto oc) {
                 constexpr int o = decltype(oc)::value;
-                if constexpr ((RLK_ABLATE & 4) != 0) {
-                } else if constexpr (o == 0 || o > TN) {
+                if constexpr (o == 0 || o > TN) {
                     constexpr int fi = o == 0 ? 0 : o - TN;
                     fa[setn][fi] = IOA::frag(rsrc, wm * (TM * 32) + fi * 32, kkn);
                 } else {
@@ -352,16 +343,14 @@ struct TileGemm {
             // right after it, so loads are spaced evenly and get a full K step of latency
             if constexpr (slot % SP == 0 && slot / SP < NW) {
                 constexpr int w = slot / SP;
-                if constexpr ((RLK_ABLATE & 2) != 0) {
-                } else if constexpr (w < PA)
+                if constexpr (w < PA)
                     la.template store_one<CHECKED>(nxt, ra, w, kstore, K);
                 else
                     lb.template store_one<CHECKED>(nxt + IOA::G::kBytes, rb, w - PA, kstore, K);
             }
             if constexpr (slot % SP == 1 && slot / SP < NW) {
                 constexpr int g = slot / SP;
-                if constexpr ((RLK_ABLATE & 1) != 0) {
-                } else if constexpr (g < PA)
+                if constexpr (g < PA)
                     la.template load_one<CHECKED>(kload, K, ra, g);
                 else
                     lb.template load_one<CHECKED>(kload, K, rb, g - PA);
@@ -412,14 +401,8 @@ struct TileGemm {
                 slice<decltype(kc)::value, CHECKED>(la, lb, ra, rb, fa, fb, wm, wn, kstore, kload, K,
                                                     cur, nxt, acc);
             });
-            if constexpr ((RLK_ABLATE & 8) == 0) __syncthreads();
+            __syncthreads();
             slice<KK - 1, CHECKED>(la, lb, ra, rb, fa, fb, wm, wn, kstore, kload, K, cur, nxt, acc);
-        }
-        if constexpr ((RLK_ABLATE & 16) != 0) {  // keep the (unused) global loads alive
-#pragma unroll
-            for (int p = 0; p < PA; ++p) asm volatile("" ::"v"(ra[p]));
-#pragma unroll
-            for (int p = 0; p < PB; ++p) asm volatile("" ::"v"(rb[p]));
         }
         __syncthreads();  // LDS may be reused by the caller
     }
@@ -478,8 +461,6 @@ struct DtlIO {
         base = reinterpret_cast<const char*>(op.base);
         next = base;
         nk = K / BK;
-        next = base;
-        nk = K / BK;
         const uint32_t ld = static_cast<uint32_t>(op.ld);
         step = KMAJOR ? static_cast<uint32_t>(BK) * ld * 2u : static_cast<uint32_t>(BK) * 2u;
 #pragma unroll
@@ -506,7 +487,6 @@ struct DtlIO {
     // the main loop waits explicitly (s_waitcnt vmcnt) before the barrier that publishes a stage.
     __device__ inline void load_one(int kt, char* lds, int p) const
     {
-        if constexpr ((RLK_ABLATE & 128) != 0) kt &= 1;  // dev: every K step re-reads cached lines
         // K steps past the end of this tile are the first steps of the next one (all uniform)
         const bool over = kt >= nk;
         const int rel = over ? (kt - nk < nk ? kt - nk : nk - 1) : kt;
@@ -561,7 +541,8 @@ struct TileGemmDtl {
 
     // Load j of a K step is issued after MFMA slot j * (LW*NM) / NL of the window that starts at
     // the last slice of the previous step.
-    template <int KKI>
+    // SKIP: the non-last slices issue no loads (the K step they would fetch is already on its way).
+    template <int KKI, bool SKIP = false>
     __device__ static inline void slice(const IOA& la, const IOB& lb, u32x4_t (&fa)[2][TM],
                                         u32x4_t (&fb)[2][TN], int wm, int wn, int kt,
                                         char* cur, char* nxt, f32x16_t (&acc)[TM][TN])
@@ -590,7 +571,7 @@ struct TileGemmDtl {
                     fb[setn][fj] = IOB::frag(rsrc + IOA::kBytes, wn * (TN * 32) + fj * 32, kkn);
                 }
             });
-            if constexpr (wslice < LW) {
+            if constexpr (wslice < LW && !(SKIP && !last)) {
                 constexpr int wslot = wslice * NM + q;
                 constexpr int lo = (wslot * NL + LW * NM - 1) / (LW * NM);        // ceil
                 constexpr int hi = ((wslot + 1) * NL + LW * NM - 1) / (LW * NM);  // ceil
@@ -600,8 +581,7 @@ struct TileGemmDtl {
                     // other slices: remaining loads of step kt+1 into the other buffer
                     const int ks = last ? kt + 2 : kt + 1;  // past the end = next tile (load_one)
                     char* dst = last ? cur : nxt;
-                    if constexpr ((RLK_ABLATE & 64) != 0) {  // dev: time without global loads
-                    } else if constexpr (g < PA)
+                    if constexpr (g < PA)
                         la.load_one(ks, dst, g);
                     else
                         lb.load_one(ks, dst + IOA::kBytes, g - PA);
@@ -620,6 +600,7 @@ struct TileGemmDtl {
         u32x4_t fa[2][TM];
         u32x4_t fb[2][TN];
         int wm, wn, nk, phase;
+        bool ahead;  // every load of the current tile's K step 1 was issued by fetch_ahead()
     };
 
     // Fill the pipeline for the first tile: K step 0 in LDS and published, the fragments of its
@@ -634,6 +615,7 @@ struct TileGemmDtl {
         st.lb.init(B, K);
         st.nk = K / BK;
         st.phase = 0;
+        st.ahead = false;
         static_for<0, PA>([&](auto pc) { st.la.load_one(0, smem, decltype(pc)::value); });
         static_for<0, PB>(
             [&](auto pc) { st.lb.load_one(0, smem + IOA::kBytes, decltype(pc)::value); });
@@ -660,13 +642,50 @@ struct TileGemmDtl {
     // the tile that follows (same leading dimensions and row counts; pass the current origins
     // after the last tile: the extra fetches then stay inside the same tile).  On return the
     // stream stands at the start of that tile exactly as begin() leaves it.
+    // REFETCH: the fragments of the first slice are read again from LDS here instead of being
+    // carried in registers from the previous tile's last slice; callers with a register-hungry
+    // epilogue between tiles use it (the K step they come from is already published).
+    // YOUNGER: after fetch_ahead() the caller's epilogue issued at least this many vector-memory
+    // instructions per wavefront (stores that may still be in flight).  The counter retires in
+    // issue order, so the first K step only has to wait until at most YOUNGER operations are
+    // outstanding to know that its own loads, which are older, have landed; the stores drain
+    // under the MFMAs instead of in front of the barrier.  A value below the true count is safe.
+    // `counted` (uniform) says whether that promise holds for the epilogue that just ran.
+    template <bool REFETCH = false, int YOUNGER = 0>
     __device__ static inline void tile(Stream& st, const void* next_a, const void* next_b,
-                                       f32x16_t (&acc)[TM][TN], char* smem)
+                                       f32x16_t (&acc)[TM][TN], char* smem, bool counted = false)
     {
         st.la.next = reinterpret_cast<const char*>(next_a);
         st.lb.next = reinterpret_cast<const char*>(next_b);
         const int nk = st.nk;
-        for (int kt = 0; kt < nk; ++kt) {
+        if constexpr (REFETCH) {
+            const char* cur0 = smem + (st.phase & 1) * kStageBytes;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) st.fa[0][i] = IOA::frag(cur0, st.wm * (TM * 32) + i * 32, 0);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                st.fb[0][j] = IOB::frag(cur0 + IOA::kBytes, st.wn * (TN * 32) + j * 32, 0);
+        }
+        int kt = 0;
+        if (st.ahead) {  // uniform: K step 1 is already on its way, issue nothing for it
+            char* cur = smem + (st.phase & 1) * kStageBytes;
+            char* nxt = smem + ((st.phase + 1) & 1) * kStageBytes;
+            static_for<0, KK - 1>([&](auto kc) {
+                slice<decltype(kc)::value, true>(st.la, st.lb, st.fa, st.fb, st.wm, st.wn, 0, cur,
+                                                 nxt, acc);
+            });
+            constexpr int wait_older = vmcnt_imm(YOUNGER < 63 ? YOUNGER : 63);
+            constexpr int wait_every = vmcnt_imm(0);
+            if (YOUNGER > 0 && counted)
+                __builtin_amdgcn_s_waitcnt(wait_older);
+            else
+                __builtin_amdgcn_s_waitcnt(wait_every);
+            __syncthreads();
+            slice<KK - 1>(st.la, st.lb, st.fa, st.fb, st.wm, st.wn, 0, cur, nxt, acc);
+            st.ahead = false;
+            kt = 1;
+        }
+        for (; kt < nk; ++kt) {
             char* cur = smem + ((kt + st.phase) & 1) * kStageBytes;
             char* nxt = smem + ((kt + st.phase + 1) & 1) * kStageBytes;
             static_for<0, KK - 1>([&](auto kc) {
@@ -681,6 +700,24 @@ struct TileGemmDtl {
         st.phase = (st.phase + nk) & 1;
         st.la.base = st.la.next;
         st.lb.base = st.lb.next;
+    }
+
+    // Call right after tile() when an epilogue with stores follows and another tile comes after
+    // it: issues now the loads of that tile's K step 1 which its first K step would otherwise
+    // issue behind the epilogue's stores (the head of the step is already in flight, the LDS stage
+    // is free since the last barrier).  The next tile() then waits with a counted vmcnt.
+    __device__ static inline void fetch_ahead(Stream& st, char* smem)
+    {
+        constexpr int first = (NM * NL + LW * NM - 1) / (LW * NM);  // loads of window slice 0
+        char* dst = smem + ((st.phase + 1) & 1) * kStageBytes;
+        static_for<first, NL>([&](auto lc) {
+            constexpr int g = decltype(lc)::value;
+            if constexpr (g < PA)
+                st.la.load_one(1, dst, g);
+            else
+                st.lb.load_one(1, dst + IOA::kBytes, g - PA);
+        });
+        st.ahead = true;
     }
 
     // Drain the fetches issued for a tile that will not be computed; LDS is free afterwards.

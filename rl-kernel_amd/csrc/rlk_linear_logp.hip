@@ -282,110 +282,185 @@ struct DzArgs {
     float scale2;
 };
 
-// Row pitch of the dZ tile staged in LDS: 512 bytes of data + 8, so that the 32 lanes of a half
-// wavefront (32 tokens, same vocab column) write 8 bytes each into distinct bank pairs.
-constexpr int kDzPitch = 520;
+// Tiles of a launch are handed out round by round: workgroup b computes the tiles with linear ids
+// b, b + gridDim.x, b + 2 gridDim.x, ...  With a grid that is a multiple of 8, a workgroup keeps
+// its XCD from round to round, so every round forms the same L2-sharing patches as a launch with
+// one workgroup per tile would.
+struct TileWalk {
+    int lin, total, gm, gn;
+    __device__ inline TileWalk(int total_, int gm_, int gn_)
+        : lin(blockIdx.x), total(total_), gm(gm_), gn(gn_) {}
+    __device__ inline bool valid() const { return lin < total; }
+    __device__ inline bool has_next() const { return lin + static_cast<int>(gridDim.x) < total; }
+    __device__ inline void coords(bool next, int& tm, int& tn) const
+    {
+        xcd_tile(next ? lin + static_cast<int>(gridDim.x) : lin, total, gm, gn, 8, tm, tn);
+    }
+    __device__ inline void advance() { lin += static_cast<int>(gridDim.x); }
+};
 
-// GENERAL = false: no bias, every vocab tile of the launch is full.
-template <class T, int BK, bool GENERAL>
-__global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
+__device__ inline void zero_acc(f32x16_t (&acc)[kTM][kTN])
+{
+#pragma unroll
+    for (int i = 0; i < kTM; ++i)
+#pragma unroll
+        for (int j = 0; j < kTN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+}
+
+// LDS each wavefront needs to turn its part of a dZ tile into full rows: 64 tokens x 32 vocab
+// columns of 16-bit values, 64 bytes per token row, no padding.
+constexpr int kDzStageBytes = 64 * 64;
+// Global stores one wavefront issues per dZ tile (kTM groups x 8 row batches), all unconditional.
+constexpr int kDzStores = kTM * 8;
+
+// dZ epilogue of one 256 x 256 tile.  A wavefront owns 128 vocab rows x 64 tokens of the tile; for
+// each of its four 32-row groups it writes the rounded values into its private LDS patch as
+// [token][vocab] rows and reads them back row-wise, so that the tile leaves in runs of 64
+// contiguous bytes per token.  Only the wavefront itself touches its patch: no workgroup barrier.
+// The 8-byte units of a row are XOR-swizzled with (token / 4) & 7, which makes both the writes
+// (32 tokens, same unit) and the reads (4 rows x 8 units) conflict-free.
+template <class T, bool GENERAL>
+__device__ inline void dz_epilogue(const f32x16_t (&acc)[kTM][kTN], const DzArgs& a, int vt, int tt,
+                                   char* stage)
 {
     constexpr int TM = kTM, TN = kTN;
-    using Gemm = TileGemm<T, false, false, BK>;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    int vt, tt;
-    xcd_tile(blockIdx.x, a.tok_tiles * a.v_tiles, a.v_tiles, a.tok_tiles, 8, vt, tt);
-    vt += a.v_tile_lo;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
     const int tok0 = tt * 256, v0 = vt * 256;
     const int tok_rows = min(256, a.tok_valid - tok0);
-    const int v_rows = min(256, a.v_valid - v0);
-
-    Operand A{a.weight + static_cast<int64_t>(v0) * a.H, a.H, v_rows};
-    Operand B{a.hidden + static_cast<int64_t>(tok0) * a.H, a.H, tok_rows};
-    f32x16_t acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    static_assert(256 * kDzPitch <= Gemm::kSmemBytes, "staged dZ tile must fit the GEMM's LDS");
-    Gemm::run(A, B, a.H, acc, smem);
-    if constexpr ((RLK_ABLATE & 32) != 0) { if (a.tok_valid >= 0) return; }  // dev: time without epilogue
-
     const float gscale = a.scales[0];
     const int vw = v0 + wm * (TM * 32);
+    const int hi = lane >> 5;
+
+    float gs[TN], nlse2[TN];
+    int etgt[TN];  // register index (i*16 + r) of the target row in this lane, or -1
+    bool any_target = false;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int tl = wn * (TN * 32) + j * 32 + (lane & 31);
         const int tc = tok0 + (tl < tok_rows ? tl : tok_rows - 1);
         const int64_t tg = a.targets[tc];
         const bool live = tl < tok_rows && !(a.use_ignore && tg == a.ignore_index);
-        const float gs = live ? a.grad[tc] * gscale : 0.f;
-        const float nlse2 = -a.lse[tc] * kLog2e;
-        // register index (i*16 + r) of the target row in this lane, or -1
+        gs[j] = live ? a.grad[tc] * gscale : 0.f;
+        nlse2[j] = -a.lse[tc] * kLog2e;
         const int64_t trel = tg - a.v_global0 - vw;
         const int tr = (trel >= 0 && trel < TM * 32) ? static_cast<int>(trel) : -1;
         const int x = tr & 31;
-        const int etgt = (tr >= 0 && ((x >> 2) & 1) == (lane >> 5))
-                             ? ((tr >> 5) * 16 + (x >> 3) * 4 + (x & 3))
-                             : -1;
-        // the 16-bit tile is staged in LDS as [token][vocab] rows so that it leaves in full lines
-        char* srow = smem + tl * kDzPitch + (wm * (TM * 32) + 4 * (lane >> 5)) * 2;
-        auto prob = [&](int i, int r) -> float {
-            float z = acc[i][j][r];
-            if (GENERAL) {
-                const int v = vw + i * 32 + acc_row(r, lane);
-                if (a.bias != nullptr) z += a.bias[v < a.v_valid ? v : a.v_valid - 1];
-                return v < a.v_valid ? __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2)) : 0.f;
-            }
-            return __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2));
-        };
-        // the one-hot term is added only when some lane of the wavefront owns its target row in
-        // this slab; values are rounded and packed two at a time
-        if (__builtin_amdgcn_ballot_w64(etgt >= 0) != 0) {  // uniform
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    float d[4];
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const int r = q * 4 + c;
-                        const float hit = (etgt == i * 16 + r) ? gs : 0.f;
-                        d[c] = fmaf(-gs, prob(i, r), hit);
-                    }
-                    *reinterpret_cast<u32x2_t*>(srow + (i * 32 + 8 * q) * 2) =
-                        u32x2_t{T::pack2(d[0], d[1]), T::pack2(d[2], d[3])};
-                }
-        } else {
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float d0 = -gs * prob(i, q * 4 + 0), d1 = -gs * prob(i, q * 4 + 1);
-                    const float d2 = -gs * prob(i, q * 4 + 2), d3 = -gs * prob(i, q * 4 + 3);
-                    *reinterpret_cast<u32x2_t*>(srow + (i * 32 + 8 * q) * 2) =
-                        u32x2_t{T::pack2(d0, d1), T::pack2(d2, d3)};
-                }
-        }
+        etgt[j] = (tr >= 0 && ((x >> 2) & 1) == hi) ? ((tr >> 5) * 16 + (x >> 3) * 4 + (x & 3)) : -1;
+        any_target = any_target || etgt[j] >= 0;
     }
-    __syncthreads();
-    // copy-out: a half wavefront moves one 512-byte row (4 full lines) as two runs of 32 x 8
-    // consecutive bytes (consecutive lanes read consecutive LDS banks)
-    uint16_t* dtile = a.dz + static_cast<int64_t>(tok0) * a.ldz + v0;
-#pragma unroll 4
-    for (int it = 0; it < 256 / (2 * (kThreads / 64)); ++it) {
-        const int row = it * (2 * (kThreads / 64)) + 2 * wave + (lane >> 5);
-        const char* src = smem + row * kDzPitch + (lane & 31) * 8;  // 8-byte aligned (pitch)
-        const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(src);
-        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(src + 256);
-        uint16_t* dst = dtile + static_cast<int64_t>(row) * a.ldz + (lane & 31) * 4;
-        *reinterpret_cast<u32x2_t*>(dst) = lo;
-        *reinterpret_cast<u32x2_t*>(dst + 128) = hi;
+    // the one-hot term is added only when some lane of the wavefront owns its target row here
+    const bool hot = __builtin_amdgcn_ballot_w64(any_target) != 0;  // uniform
+
+    uint16_t* dtile = a.dz + static_cast<int64_t>(tok0 + wn * (TN * 32)) * a.ldz + vw;
+    auto stage_rows = [&](auto ic, auto hot_c) {
+        constexpr int i = decltype(ic)::value;
+        constexpr bool HOT = decltype(hot_c)::value;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int t = j * 32 + (lane & 31);  // token row inside the wavefront's patch
+            char* srow = stage + t * 64;
+            const int sw = (t >> 2) & 7;
+            auto prob = [&](int r) -> float {
+                float z = acc[i][j][r];
+                if (GENERAL) {
+                    const int v = vw + i * 32 + acc_row(r, lane);
+                    if (a.bias != nullptr) z += a.bias[v < a.v_valid ? v : a.v_valid - 1];
+                    return v < a.v_valid ? __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2[j])) : 0.f;
+                }
+                return __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2[j]));
+            };
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float d[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if constexpr (HOT) {
+                        const float hit = (etgt[j] == i * 16 + q * 4 + c) ? gs[j] : 0.f;
+                        d[c] = fmaf(-gs[j], prob(q * 4 + c), hit);
+                    } else {
+                        d[c] = -gs[j] * prob(q * 4 + c);
+                    }
+                }
+                // rows 8q + 4hi + 0..3 of this 32-row group: unit 2q + hi of the token's row
+                *reinterpret_cast<u32x2_t*>(srow + (((2 * q + hi) ^ sw) * 8)) =
+                    u32x2_t{T::pack2(d[0], d[1]), T::pack2(d[2], d[3])};
+            }
+        }
+    };
+    static_for<0, TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if (hot)
+            stage_rows(ic, std::true_type{});
+        else
+            stage_rows(ic, std::false_type{});
+        __builtin_amdgcn_wave_barrier();
+        // copy-out: 8 lanes move one token row (64 bytes), 8 rows per instruction
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int row = it * 8 + (lane >> 3);
+            const int u = lane & 7;
+            const u32x2_t v = *reinterpret_cast<const u32x2_t*>(stage + row * 64 + ((u ^ ((row >> 2) & 7)) * 8));
+            *reinterpret_cast<u32x2_t*>(dtile + static_cast<int64_t>(row) * a.ldz + i * 32 + u * 4) = v;
+        }
+        __builtin_amdgcn_wave_barrier();
+    });
+}
+
+// GENERAL = false: no bias, every vocab tile of the launch is full.
+// CHAIN (needs !GENERAL, full token tiles, H a multiple of BK and >= 2 BK): the workgroup walks
+// its tiles through one pipeline; while a tile's epilogue runs, the first K steps of the next
+// tile are already on their way into LDS.
+template <class T, int BK, bool GENERAL, bool CHAIN>
+__global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
+{
+    static_assert(!(GENERAL && CHAIN), "the chained variant covers full tiles only");
+    using Gemm = TileGemm<T, false, false, BK>;
+    using Dtl = TileGemmDtl<T, false, false, BK>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int wave = threadIdx.x >> 6;
+    TileWalk walk(a.tok_tiles * a.v_tiles, a.v_tiles, a.tok_tiles);
+    if (!walk.valid()) return;
+    int vt, tt;
+    walk.coords(false, vt, tt);
+    auto w_origin = [&](int v) { return a.weight + static_cast<int64_t>(v + a.v_tile_lo) * 256 * a.H; };
+    auto h_origin = [&](int t) { return a.hidden + static_cast<int64_t>(t) * 256 * a.H; };
+    f32x16_t acc[kTM][kTN];
+    if constexpr (CHAIN) {
+        char* stage = smem + Dtl::kSmemBytes + wave * kDzStageBytes;
+        typename Dtl::Stream st;
+        Dtl::begin(st, Operand{w_origin(vt), a.H, 256}, Operand{h_origin(tt), a.H, 256}, a.H, smem);
+        for (;;) {
+            const bool more = walk.has_next();
+            int nvt = vt, ntt = tt;
+            if (more) walk.coords(true, nvt, ntt);
+            zero_acc(acc);
+            Dtl::template tile<true, kDzStores / 2>(st, w_origin(nvt), h_origin(ntt), acc, smem, true);
+            if (more) Dtl::fetch_ahead(st, smem);
+            dz_epilogue<T, GENERAL>(acc, a, vt + a.v_tile_lo, tt, stage);
+            if (!more) break;
+            walk.advance();
+            vt = nvt;
+            tt = ntt;
+        }
+        Dtl::end(st);
+    } else {
+        static_assert(kDzStageBytes * (kThreads / 64) <= Gemm::kSmemBytes, "staging must fit the GEMM's LDS");
+        for (;;) {
+            const int tok0 = tt * 256, v0 = (vt + a.v_tile_lo) * 256;
+            Operand A{w_origin(vt), a.H, min(256, a.v_valid - v0)};
+            Operand B{h_origin(tt), a.H, min(256, a.tok_valid - tok0)};
+            zero_acc(acc);
+            Gemm::run(A, B, a.H, acc, smem);  // ends with a barrier: LDS is free
+            dz_epilogue<T, GENERAL>(acc, a, vt + a.v_tile_lo, tt, smem + wave * kDzStageBytes);
+            if (!walk.has_next()) break;
+            walk.advance();
+            walk.coords(false, vt, tt);
+            __syncthreads();  // every wavefront has left its staging patch
+        }
     }
 }
 
@@ -411,97 +486,157 @@ struct DhArgs {
     int64_t part_stride;  //      (elements per slot); linear_logp_dh_reduce_kernel adds them up
 };
 
-template <class T, int BK>
-__global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
+// Epilogue of one dH tile.  The read-modify-write of the running fp32 partial is latency-bound, so
+// it runs in two batches (one per 32-token column group): the 16 reads of a batch are all issued
+// before the first use, then added and stored.  FULL (the tile lies inside the chunk and inside
+// H): addresses are a uniform tile origin plus a 32-bit lane offset and no predicates are needed;
+// otherwise rows and columns are clamped for the reads and predicated for the stores.
+template <class T, bool FULL>
+__device__ inline void dh_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const DhArgs& a, int tt,
+                                        int ht, float* acc_dst, bool first, bool last)
 {
     constexpr int TM = kTM, TN = kTN;
-    using Gemm = TileGemm<T, true, false, BK>;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    int tt, ht, ks = 0;
-    xcd_tile(blockIdx.x, a.tok_tiles * a.h_tiles * a.ksplit, a.tok_tiles, a.h_tiles * a.ksplit, 8,
-             tt, ht);
-    // K range of this workgroup: whole 64-row steps, the first (steps % ksplit) parts take one more
-    int k0 = 0, kn = a.v_valid;
-    float* acc_dst = a.acc;
-    bool first = a.first != 0, last = a.last != 0, empty_part = false;
-    if (a.ksplit > 1) {  // uniform
-        ks = ht % a.ksplit;
-        ht /= a.ksplit;
-        const int steps = (a.v_valid + BK - 1) / BK;
-        const int base = steps / a.ksplit, extra = steps % a.ksplit;
-        const int s0 = ks * base + (ks < extra ? ks : extra);
-        const int s1 = s0 + base + (ks < extra ? 1 : 0);
-        k0 = s0 * BK;
-        kn = min(a.v_valid, s1 * BK) - k0;
-        if (kn <= 0) {  // a short last piece can leave a part without K steps: it computes one
-            empty_part = true;  // step of the piece's head and discards it
-            k0 = 0;
-            kn = min(a.v_valid, BK);
-        }
-        acc_dst = a.part + static_cast<int64_t>(ks) * a.part_stride;
-        first = true;
-        last = false;
-    }
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
     const int tok0 = tt * 256, h0 = ht * 256;
-
-    Operand A{a.weight + static_cast<int64_t>(k0) * a.H + h0, a.H, min(256, a.H - h0)};
-    Operand B{a.dz + static_cast<int64_t>(tok0) * a.ldz + k0, a.ldz, 256};
-    f32x16_t acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    Gemm::run(A, B, kn, acc, smem);
-    if (empty_part) {  // uniform: this part's slot must hold zeros
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    }
-    if constexpr ((RLK_ABLATE & 32) != 0) { if (a.tok_valid >= 0) return; }  // dev: time without epilogue
-
-    // Epilogue: all reads of the running fp32 partial are issued before the first use (clamped
-    // addresses instead of branches), then added and stored under a predicate.
     const float oscale = a.scales[1];
+    const int hbase = h0 + wm * (TM * 32) + 4 * (lane >> 5);  // + i * 32 + 8 * q
+    const uint32_t ldh = static_cast<uint32_t>(a.H);
+    // FULL: byte offsets inside the tile stay below 256 * H * 4 (32 bits)
+    const int64_t origin = static_cast<int64_t>(tok0) * a.H + h0;
+    char* acc_tile = reinterpret_cast<char*>(acc_dst + origin);
+    char* out_tile = reinterpret_cast<char*>(a.out + origin);
+    const uint32_t lane_el = static_cast<uint32_t>(wn * (TN * 32) + (lane & 31)) * ldh +
+                             static_cast<uint32_t>(wm * (TM * 32) + 4 * (lane >> 5));
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int tl = tok0 + wn * (TN * 32) + j * 32 + (lane & 31);
-        const bool tok_ok = tl < a.tok_valid;
+        const bool tok_ok = FULL || tl < a.tok_valid;
         const int64_t trow = static_cast<int64_t>(tok_ok ? tl : a.tok_valid - 1) * a.H;
+        f32x4_t old[TM][4];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            f32x4_t old[4];
-            int hcol[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int h = h0 + wm * (TM * 32) + i * 32 + 8 * q + 4 * (lane >> 5);
-                hcol[q] = h;
-                old[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-                if (!first)  // uniform
-                    old[q] = *reinterpret_cast<const f32x4_t*>(acc_dst + trow + (h < a.H ? h : 0));
-            }
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                f32x4_t v{acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
-                          acc[i][j][q * 4 + 3]};
-                v += old[q];
-                if (tok_ok && hcol[q] < a.H) {  // H % 8 == 0: a quad is all-in or all-out
-                    if (last) {
-                        u32x2_t pk{T::pack2(v.x * oscale, v.y * oscale), T::pack2(v.z * oscale, v.w * oscale)};
-                        *reinterpret_cast<u32x2_t*>(a.out + trow + hcol[q]) = pk;
+                old[i][q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                if (!first) {  // uniform
+                    if (FULL) {
+                        const char* rowp = acc_tile + (static_cast<size_t>(j * 32) * ldh + (i * 32 + 8 * q)) * 4u;
+                        old[i][q] = *reinterpret_cast<const f32x4_t*>(rowp + lane_el * 4u);
                     } else {
-                        *reinterpret_cast<f32x4_t*>(acc_dst + trow + hcol[q]) = v;
+                        const int h = hbase + i * 32 + 8 * q;
+                        old[i][q] = *reinterpret_cast<const f32x4_t*>(acc_dst + trow + (h < a.H ? h : 0));
                     }
                 }
             }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int h = hbase + i * 32 + 8 * q;
+                f32x4_t v{acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                          acc[i][j][q * 4 + 3]};
+                v += old[i][q];
+                const size_t uni = static_cast<size_t>(j * 32) * ldh + (i * 32 + 8 * q);  // uniform
+                if (FULL || (tok_ok && h < a.H)) {  // H % 8 == 0: a quad is all-in or all-out
+                    if (last) {
+                        u32x2_t pk{T::pack2(v.x * oscale, v.y * oscale), T::pack2(v.z * oscale, v.w * oscale)};
+                        if (FULL)
+                            *reinterpret_cast<u32x2_t*>(out_tile + uni * 2u + lane_el * 2u) = pk;
+                        else
+                            *reinterpret_cast<u32x2_t*>(a.out + trow + h) = pk;
+                    } else {
+                        if (FULL)
+                            *reinterpret_cast<f32x4_t*>(acc_tile + uni * 4u + lane_el * 4u) = v;
+                        else
+                            *reinterpret_cast<f32x4_t*>(acc_dst + trow + h) = v;
+                    }
+                }
+            }
+    }
+}
+
+// Returns whether the tile was full (then every wavefront issued all its stores unconditionally).
+template <class T>
+__device__ inline bool dh_epilogue(const f32x16_t (&acc)[kTM][kTN], const DhArgs& a, int tt, int ht,
+                                   float* acc_dst, bool first, bool last)
+{
+    const bool full = tt * 256 + 256 <= a.tok_valid && ht * 256 + 256 <= a.H;  // uniform
+    if (full)
+        dh_epilogue_impl<T, true>(acc, a, tt, ht, acc_dst, first, last);
+    else
+        dh_epilogue_impl<T, false>(acc, a, tt, ht, acc_dst, first, last);
+    return full;
+}
+
+// CHAIN (needs ksplit == 1, H a multiple of 256, v_valid a multiple of BK and >= 2 BK): the
+// workgroup walks its tiles through one pipeline.
+template <class T, int BK, bool CHAIN>
+__global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
+{
+    using Gemm = TileGemm<T, true, false, BK>;
+    using Dtl = TileGemmDtl<T, true, false, BK>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    f32x16_t acc[kTM][kTN];
+    if constexpr (CHAIN) {
+        TileWalk walk(a.tok_tiles * a.h_tiles, a.tok_tiles, a.h_tiles);
+        if (!walk.valid()) return;
+        int tt, ht;
+        walk.coords(false, tt, ht);
+        auto w_origin = [&](int h) { return a.weight + static_cast<int64_t>(h) * 256; };
+        auto z_origin = [&](int t) { return a.dz + static_cast<int64_t>(t) * 256 * a.ldz; };
+        typename Dtl::Stream st;
+        bool counted = false;
+        Dtl::begin(st, Operand{w_origin(ht), a.H, 256}, Operand{z_origin(tt), a.ldz, 256}, a.v_valid, smem);
+        for (;;) {
+            const bool more = walk.has_next();
+            int ntt = tt, nht = ht;
+            if (more) walk.coords(true, ntt, nht);
+            zero_acc(acc);
+            // a full tile's epilogue issues kTM * kTN * 4 unconditional stores per wavefront
+            Dtl::template tile<true, kTM * kTN * 2>(st, w_origin(nht), z_origin(ntt), acc, smem, counted);
+            if (more) Dtl::fetch_ahead(st, smem);
+            counted = dh_epilogue<T>(acc, a, tt, ht, a.acc, a.first != 0, a.last != 0);
+            if (!more) break;
+            walk.advance();
+            tt = ntt;
+            ht = nht;
         }
+        Dtl::end(st);
+    } else {
+        int tt, ht, ks = 0;
+        xcd_tile(blockIdx.x, a.tok_tiles * a.h_tiles * a.ksplit, a.tok_tiles, a.h_tiles * a.ksplit, 8,
+                 tt, ht);
+        // K range of this workgroup: whole BK-row steps, the first (steps % ksplit) parts take one more
+        int k0 = 0, kn = a.v_valid;
+        float* acc_dst = a.acc;
+        bool first = a.first != 0, last = a.last != 0, empty_part = false;
+        if (a.ksplit > 1) {  // uniform
+            ks = ht % a.ksplit;
+            ht /= a.ksplit;
+            const int steps = (a.v_valid + BK - 1) / BK;
+            const int base = steps / a.ksplit, extra = steps % a.ksplit;
+            const int s0 = ks * base + (ks < extra ? ks : extra);
+            const int s1 = s0 + base + (ks < extra ? 1 : 0);
+            k0 = s0 * BK;
+            kn = min(a.v_valid, s1 * BK) - k0;
+            if (kn <= 0) {  // a short last piece can leave a part without K steps: it computes one
+                empty_part = true;  // step of the piece's head and discards it
+                k0 = 0;
+                kn = min(a.v_valid, BK);
+            }
+            acc_dst = a.part + static_cast<int64_t>(ks) * a.part_stride;
+            first = true;
+            last = false;
+        }
+        const int tok0 = tt * 256, h0 = ht * 256;
+        Operand A{a.weight + static_cast<int64_t>(k0) * a.H + h0, a.H, min(256, a.H - h0)};
+        Operand B{a.dz + static_cast<int64_t>(tok0) * a.ldz + k0, a.ldz, 256};
+        zero_acc(acc);
+        Gemm::run(A, B, kn, acc, smem);
+        if (empty_part) zero_acc(acc);  // uniform: this part's slot must hold zeros
+        dh_epilogue<T>(acc, a, tt, ht, acc_dst, first, last);
     }
 }
 
@@ -528,7 +663,7 @@ __global__ void linear_logp_dh_reduce_kernel(const float* part, int ksplit, int6
 }
 
 // ------------------------------------------------------------------------------------------- //
-// Backward step 3: dW[v][h] (+)= sum_tok dZ[tok][v] hidden[tok][h]   (M = vocab, N = h, K = token)
+// Backward step 3: dW[v][h] (+)= sum_tok dZ[tok][v] hidden[tok][h]   (M = h, N = vocab, K = token)
 // ------------------------------------------------------------------------------------------- //
 struct DwArgs {
     const uint16_t* dz;      // [tok_tiles*256][ldz]
@@ -544,55 +679,121 @@ struct DwArgs {
     int accumulate;  // 1: dw += ..., 0: dw = ...
 };
 
-template <class T, int BK>
-__global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
+// Epilogue of one dW tile.  Orientation: M (accumulator registers) = hidden column, N (lane) =
+// vocab row, so a lane holds 4 consecutive columns of one dW row and the read-modify-write of the
+// fp32 tile moves 16 bytes per lane.  It is latency-bound and therefore runs in two batches (one
+// per 32-row group): the 16 reads of a batch are issued before the first use.  FULL (the tile lies
+// inside the piece and inside H): a uniform tile origin plus a 32-bit lane offset, no predicates;
+// otherwise clamped reads and predicated stores.
+template <bool FULL>
+__device__ inline void dw_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const DwArgs& a, int vt, int ht)
 {
     constexpr int TM = kTM, TN = kTN;
-    using Gemm = TileGemm<T, true, true, BK>;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    int vt, ht;
-    xcd_tile(blockIdx.x, a.v_tiles * a.h_tiles, a.v_tiles, a.h_tiles, 8, vt, ht);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
     const int v0 = vt * 256, h0 = ht * 256;
-
-    Operand A{a.dz + v0, a.ldz, 256};
-    Operand B{a.hidden + h0, a.H, min(256, a.H - h0)};
-    f32x16_t acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    Gemm::run(A, B, a.tok_valid, acc, smem);
-    if constexpr ((RLK_ABLATE & 32) != 0) { if (a.tok_valid >= 0) return; }  // dev: time without epilogue
-
-    // Epilogue: read-modify-write of the fp32 dW tile; the 16 reads of one MFMA tile are issued
-    // together (clamped addresses), then added and stored under a predicate.
     const float oscale = a.scales[1];
+    const int hbase = h0 + wm * (TM * 32) + 4 * (lane >> 5);  // + i * 32 + 8 * q
+    const uint32_t ldw = static_cast<uint32_t>(a.H);
+    // FULL: byte offsets inside the tile stay below 256 * H * 4 (32 bits)
+    char* tile = reinterpret_cast<char*>(a.dw + static_cast<int64_t>(v0) * a.H + h0);
+    const uint32_t lane_el = static_cast<uint32_t>(wn * (TN * 32) + (lane & 31)) * ldw +
+                             static_cast<uint32_t>(wm * (TM * 32) + 4 * (lane >> 5));
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int h = h0 + wn * (TN * 32) + j * 32 + (lane & 31);
-        const bool h_ok = h < a.H;
-        const int hc = h_ok ? h : 0;
+        const int v = v0 + wn * (TN * 32) + j * 32 + (lane & 31);
+        const bool v_ok = FULL || v < a.v_valid;
+        const int64_t vrow = static_cast<int64_t>(v_ok ? v : a.v_valid - 1) * a.H;
+        f32x4_t old[TM][4];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            float old[16];
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int v = v0 + wm * (TM * 32) + i * 32 + acc_row(r, lane);
-                old[r] = 0.f;
-                if (a.accumulate)  // uniform
-                    old[r] = a.dw[static_cast<int64_t>(v < a.v_valid ? v : a.v_valid - 1) * a.H + hc];
+            for (int q = 0; q < 4; ++q) {
+                old[i][q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                if (a.accumulate) {  // uniform
+                    if (FULL) {
+                        const char* rowp = tile + (static_cast<size_t>(j * 32) * ldw + (i * 32 + 8 * q)) * 4u;
+                        old[i][q] = *reinterpret_cast<const f32x4_t*>(rowp + lane_el * 4u);
+                    } else {
+                        const int h = hbase + i * 32 + 8 * q;
+                        old[i][q] = *reinterpret_cast<const f32x4_t*>(a.dw + vrow + (h < a.H ? h : 0));
+                    }
+                }
             }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int v = v0 + wm * (TM * 32) + i * 32 + acc_row(r, lane);
-                if (h_ok && v < a.v_valid)
-                    a.dw[static_cast<int64_t>(v) * a.H + h] = fmaf(acc[i][j][r], oscale, old[r]);
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int h = hbase + i * 32 + 8 * q;
+                f32x4_t val{acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                            acc[i][j][q * 4 + 3]};
+                val = val * oscale + old[i][q];
+                if (FULL) {
+                    char* rowp = tile + (static_cast<size_t>(j * 32) * ldw + (i * 32 + 8 * q)) * 4u;
+                    *reinterpret_cast<f32x4_t*>(rowp + lane_el * 4u) = val;
+                } else if (v_ok && h < a.H) {  // H % 8 == 0: a quad is all-in or all-out
+                    *reinterpret_cast<f32x4_t*>(a.dw + vrow + h) = val;
+                }
             }
+    }
+}
+
+// Returns whether the tile was full (then every wavefront issued all its stores unconditionally).
+__device__ inline bool dw_epilogue(const f32x16_t (&acc)[kTM][kTN], const DwArgs& a, int vt, int ht)
+{
+    const bool full = vt * 256 + 256 <= a.v_valid && ht * 256 + 256 <= a.H;  // uniform
+    if (full)
+        dw_epilogue_impl<true>(acc, a, vt, ht);
+    else
+        dw_epilogue_impl<false>(acc, a, vt, ht);
+    return full;
+}
+
+// CHAIN (needs H a multiple of 256, tok_valid a multiple of BK and >= 2 BK): the workgroup walks
+// its tiles through one pipeline.
+template <class T, int BK, bool CHAIN>
+__global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
+{
+    using Gemm = TileGemm<T, true, true, BK>;
+    using Dtl = TileGemmDtl<T, true, true, BK>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    TileWalk walk(a.v_tiles * a.h_tiles, a.v_tiles, a.h_tiles);
+    if (!walk.valid()) return;
+    int vt, ht;
+    walk.coords(false, vt, ht);
+    f32x16_t acc[kTM][kTN];
+    auto h_origin = [&](int h) { return a.hidden + static_cast<int64_t>(h) * 256; };  // M rows
+    auto z_origin = [&](int v) { return a.dz + static_cast<int64_t>(v) * 256; };      // N rows
+    if constexpr (CHAIN) {
+        typename Dtl::Stream st;
+        bool counted = false;
+        Dtl::begin(st, Operand{h_origin(ht), a.H, 256}, Operand{z_origin(vt), a.ldz, 256}, a.tok_valid, smem);
+        for (;;) {
+            const bool more = walk.has_next();
+            int nvt = vt, nht = ht;
+            if (more) walk.coords(true, nvt, nht);
+            zero_acc(acc);
+            // a full tile's epilogue issues kTM * kTN * 4 unconditional stores per wavefront
+            Dtl::template tile<true, kTM * kTN * 2>(st, h_origin(nht), z_origin(nvt), acc, smem, counted);
+            if (more) Dtl::fetch_ahead(st, smem);
+            counted = dw_epilogue(acc, a, vt, ht);
+            if (!more) break;
+            walk.advance();
+            vt = nvt;
+            ht = nht;
+        }
+        Dtl::end(st);
+    } else {
+        for (;;) {
+            Operand A{h_origin(ht), a.H, min(256, a.H - ht * 256)};
+            Operand B{z_origin(vt), a.ldz, 256};
+            zero_acc(acc);
+            Gemm::run(A, B, a.tok_valid, acc, smem);
+            dw_epilogue(acc, a, vt, ht);
+            if (!walk.has_next()) break;
+            walk.advance();
+            walk.coords(false, vt, ht);
         }
     }
 }
@@ -677,6 +878,22 @@ namespace {
 
 constexpr int kBK = RLK_BK;
 
+// 1: backward launches whose tiles are all full run one persistent workgroup per compute unit
+// that chains its tiles through one pipeline; 0: one workgroup per tile everywhere.
+#ifndef RLK_CHAIN
+#define RLK_CHAIN 1
+#endif
+#ifndef RLK_CHAIN_DH
+#define RLK_CHAIN_DH RLK_CHAIN
+#endif
+#ifndef RLK_CHAIN_DW
+#define RLK_CHAIN_DW RLK_CHAIN
+#endif
+// Extra elements between token rows of the dZ block (multiple of 8).
+#ifndef RLK_LDZ_PAD
+#define RLK_LDZ_PAD 0
+#endif
+
 // Forward launch plan: a pure function of (N, V, bias present).
 //   fast launch   : full vocab tiles [0, full_tiles) split n_fast ways, no bias
 //   general launch: the remaining tiles (all tiles when there is a bias) split n_gen ways
@@ -727,6 +944,7 @@ struct BwdPlan {
     int n_chunks;
     int n_pieces;
     int ksplit;      // dH launch: parts of the piece's vocab range computed side by side
+    int64_t ldz;     // elements between consecutive token rows of the dZ block
     size_t dz_bytes;
     size_t acc_bytes;
     size_t part_bytes;
@@ -734,13 +952,15 @@ struct BwdPlan {
 };
 
 // Cost of the three launches of one dZ block of ct x pt tiles, in K steps of one CU: a launch of
-// t tiles occupies ceil(t / 256) rounds of the 256 CUs, a tile costs its K steps plus an epilogue
-// (dZ: exp + 16-bit store; dH / dW: fp32 read-modify-write of the tile).
+// t tiles occupies ceil(t / 256) rounds of the 256 CUs, a tile costs its K steps plus an epilogue.
+// Measured on MI355X with wall-clock stamps inside the kernels, one K step (256 x 256 x 64) takes
+// about 1.56 us in all three kernels; the dZ epilogue (exp + 16-bit store) 4.4 us = 3 steps, the
+// fp32 read-modify-write of a dH or dW tile 13 - 14 us = 9 steps.
 inline int64_t block_cost(int64_t ct, int64_t pt, int64_t ht, int64_t hk)
 {
-    const int64_t dz = (ct * pt + 255) / 256 * (hk + 12);
-    const int64_t dh = (ct * ht + 255) / 256 * (4 * pt + 28);
-    const int64_t dw = (pt * ht + 255) / 256 * (4 * ct + 28);
+    const int64_t dz = (ct * pt + 255) / 256 * (hk + 3);
+    const int64_t dh = (ct * ht + 255) / 256 * (4 * pt + 9);
+    const int64_t dw = (pt * ht + 255) / 256 * (4 * ct + 9);
     return dz + dh + dw;
 }
 
@@ -804,7 +1024,8 @@ BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
     p.v_piece = static_cast<int>(best_pt) * 256;
     p.n_chunks = static_cast<int>((n_t + best_ct - 1) / best_ct);
     p.n_pieces = static_cast<int>((v_t + best_pt - 1) / best_pt);
-    p.dz_bytes = static_cast<size_t>(p.tok_chunk) * p.v_piece * 2;
+    p.ldz = p.v_piece + RLK_LDZ_PAD;
+    p.dz_bytes = static_cast<size_t>(p.tok_chunk) * p.ldz * 2;
     p.acc_bytes = p.n_pieces > 1 ? static_cast<size_t>(p.tok_chunk) * H * 4 : 0;
     p.scales_off = 0;
     p.dz_off = 256;
@@ -856,6 +1077,219 @@ bool use_mfma(const void* hidden, const void* weight, int32_t H, int dtype)
 {
     return (dtype == RLK_DTYPE_BF16 || dtype == RLK_DTYPE_F16) && H % 8 == 0 &&
            (reinterpret_cast<uintptr_t>(hidden) & 15) == 0 && (reinterpret_cast<uintptr_t>(weight) & 15) == 0;
+}
+
+// Compute units of the current device (looked up once per device): the chained kernels launch
+// one workgroup per compute unit.  Which workgroup computes a tile never changes the tile's bits.
+int compute_units(int* out)
+{
+    constexpr int kMaxDev = 64;
+    static std::mutex mu;
+    static int cached[kMaxDev] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDev) return rlk_fail(RLK_ERR_UNSUPPORTED, "device index too large");
+    std::lock_guard<std::mutex> lock(mu);
+    if (cached[dev] == 0) {
+        int n = 0;
+        e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess || n <= 0) return rlk_fail(RLK_ERR_LAUNCH, "cannot read the compute-unit count");
+        cached[dev] = n;
+    }
+    *out = cached[dev];
+    return 0;
+}
+
+struct BwdCall {
+    const float* grad_logp;
+    const void* hidden;
+    const void* weight;
+    const float* bias;
+    const int64_t* targets;
+    const float* lse;
+    void* d_hidden;
+    float* d_weight;
+    float* d_bias;
+    void* workspace;
+    int64_t N;
+    int32_t H;
+    int64_t V;
+    int64_t vocab_start;
+    int32_t dtype;
+    float temperature;
+    int64_t ignore_index;
+    int32_t use_ignore;
+    hipStream_t stream;
+};
+
+// Grid of a chained launch: one workgroup per compute unit, rounded down to a multiple of 8 so
+// that a workgroup stays on one XCD from round to round; never more workgroups than tiles.
+inline int chain_grid(int tiles, int n_cu)
+{
+    int g = n_cu >= 8 ? n_cu / 8 * 8 : n_cu;
+    return tiles < g ? tiles : g;
+}
+
+// Enqueues the backward schedule: for every (token chunk, vocab piece) block
+//   dZ recompute -> dH (+)= dZ W -> dW (+)= dZ^T hidden (-> db).
+template <class T>
+int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
+{
+    using GZ = TileGemm<T, false, false, kBK>;
+    using GH = TileGemm<T, true, false, kBK>;
+    using GW = TileGemm<T, true, true, kBK>;
+    constexpr int kChainSmem = TileGemmDtl<T, false, false, kBK>::kSmemBytes;
+    constexpr int kDzChainSmem = kChainSmem + kDzStageBytes * (kThreads / 64);
+    const int H = c.H;
+    const int64_t N = c.N, V = c.V;
+    hipStream_t stream = c.stream;
+
+    char* ws = static_cast<char*>(c.workspace);
+    float* scales = reinterpret_cast<float*>(ws + p.scales_off);
+    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.dz_off);
+    float* hacc = p.acc_bytes ? reinterpret_cast<float*>(ws + p.acc_off) : nullptr;
+    const uint16_t* hid = static_cast<const uint16_t*>(c.hidden);
+    const uint16_t* w = static_cast<const uint16_t*>(c.weight);
+    uint16_t* dh = static_cast<uint16_t*>(c.d_hidden);
+    const int h_tiles = (H + 255) / 256;
+
+    hipLaunchKernelGGL(linear_logp_scales_kernel, dim3(1), dim3(1024), 0, stream, c.grad_logp,
+                       static_cast<int>(N), 1.f / c.temperature, c.dtype, scales);
+    if (int rc = check_launch("scales kernel launch failed")) return rc;
+
+    if (int rc = set_smem(linear_logp_dz_kernel<T, kBK, false, true>, kDzChainSmem)) return rc;
+    if (int rc = set_smem(linear_logp_dz_kernel<T, kBK, false, false>, GZ::kSmemBytes)) return rc;
+    if (int rc = set_smem(linear_logp_dz_kernel<T, kBK, true, false>, GZ::kSmemBytes)) return rc;
+    if (int rc = set_smem(linear_logp_dh_kernel<T, kBK, true>, kChainSmem)) return rc;
+    if (int rc = set_smem(linear_logp_dh_kernel<T, kBK, false>, GH::kSmemBytes)) return rc;
+    if (int rc = set_smem(linear_logp_dw_kernel<T, kBK, true>, kChainSmem)) return rc;
+    if (int rc = set_smem(linear_logp_dw_kernel<T, kBK, false>, GW::kSmemBytes)) return rc;
+
+    for (int ci = 0; ci < p.n_chunks; ++ci) {
+        const int64_t tok_lo = static_cast<int64_t>(ci) * p.tok_chunk;
+        const int tok_valid = static_cast<int>((N - tok_lo) < p.tok_chunk ? (N - tok_lo) : p.tok_chunk);
+        if (tok_valid <= 0) break;
+        const int tok_tiles = (tok_valid + 255) / 256;
+        for (int pi = 0; pi < p.n_pieces; ++pi) {
+            const int64_t v_lo = static_cast<int64_t>(pi) * p.v_piece;
+            const int v_valid = static_cast<int>((V - v_lo) < p.v_piece ? (V - v_lo) : p.v_piece);
+            if (v_valid <= 0) break;
+            const int v_tiles = (v_valid + 255) / 256;
+            const bool last_piece = (v_lo + p.v_piece >= V);
+
+            DzArgs z;
+            z.hidden = hid + tok_lo * H;
+            z.weight = w + v_lo * H;
+            z.bias = c.bias ? c.bias + v_lo : nullptr;
+            z.targets = c.targets + tok_lo;
+            z.lse = c.lse + tok_lo;
+            z.grad = c.grad_logp + tok_lo;
+            z.scales = scales;
+            z.dz = dz;
+            z.ldz = p.ldz;
+            z.tok_valid = tok_valid;
+            z.v_valid = v_valid;
+            z.H = H;
+            z.tok_tiles = tok_tiles;
+            z.v_global0 = c.vocab_start + v_lo;
+            z.ignore_index = c.ignore_index;
+            z.use_ignore = c.use_ignore;
+            z.scale2 = kLog2e / c.temperature;
+
+            DhArgs h;
+            h.dz = dz;
+            h.weight = w + v_lo * H;
+            h.scales = scales;
+            h.acc = hacc;
+            h.out = dh ? dh + tok_lo * H : nullptr;
+            h.ldz = p.ldz;
+            h.H = H;
+            h.v_valid = v_valid;
+            h.tok_valid = tok_valid;
+            h.tok_tiles = tok_tiles;
+            h.h_tiles = h_tiles;
+            h.first = pi == 0;
+            h.last = last_piece;
+            h.ksplit = p.ksplit;
+            h.part = p.ksplit > 1 ? reinterpret_cast<float*>(ws + p.part_off) : nullptr;
+            h.part_stride = static_cast<int64_t>(p.tok_chunk) * H;
+
+            DwArgs d;
+            d.dz = dz;
+            d.hidden = hid + tok_lo * H;
+            d.scales = scales;
+            d.dw = c.d_weight ? c.d_weight + v_lo * H : nullptr;
+            d.ldz = p.ldz;
+            d.H = H;
+            d.v_valid = v_valid;
+            d.tok_valid = tok_valid;
+            d.v_tiles = v_tiles;
+            d.h_tiles = h_tiles;
+            d.accumulate = ci > 0;
+
+            // dZ block: full vocab tiles through the fast variant (chained through one pipeline
+            // when the token tiles are full too), the rest (all of them when there is a bias)
+            // through the general one
+            const int fast_tiles = c.bias ? 0 : v_valid / 256;
+            const int gen_tiles = v_tiles - fast_tiles;
+            const bool k_ok = H % kBK == 0 && H >= 2 * kBK;
+            if (fast_tiles > 0) {
+                z.v_tiles = fast_tiles;
+                z.v_tile_lo = 0;
+                const int tiles = tok_tiles * fast_tiles;
+                if (RLK_CHAIN && k_ok && tok_valid % 256 == 0)
+                    hipLaunchKernelGGL((linear_logp_dz_kernel<T, kBK, false, true>),
+                                       dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kDzChainSmem,
+                                       stream, z);
+                else
+                    hipLaunchKernelGGL((linear_logp_dz_kernel<T, kBK, false, false>), dim3(tiles),
+                                       dim3(kThreads), GZ::kSmemBytes, stream, z);
+            }
+            if (gen_tiles > 0) {
+                z.v_tiles = gen_tiles;
+                z.v_tile_lo = fast_tiles;
+                hipLaunchKernelGGL((linear_logp_dz_kernel<T, kBK, true, false>),
+                                   dim3(tok_tiles * gen_tiles), dim3(kThreads), GZ::kSmemBytes,
+                                   stream, z);
+            }
+            if (dh) {
+                const int tiles = tok_tiles * h_tiles;
+                if (RLK_CHAIN_DH && p.ksplit == 1 && H % 256 == 0 && v_valid % kBK == 0 && v_valid >= 2 * kBK) {
+                    hipLaunchKernelGGL((linear_logp_dh_kernel<T, kBK, true>),
+                                       dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kChainSmem,
+                                       stream, h);
+                } else {
+                    hipLaunchKernelGGL((linear_logp_dh_kernel<T, kBK, false>),
+                                       dim3(tiles * p.ksplit), dim3(kThreads), GH::kSmemBytes, stream, h);
+                    if (p.ksplit > 1) {
+                        const int64_t n4 = static_cast<int64_t>(tok_valid) * H / 4;
+                        hipLaunchKernelGGL((linear_logp_dh_reduce_kernel<T>),
+                                           dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0,
+                                           stream, h.part, p.ksplit, h.part_stride, h.acc, h.out,
+                                           scales, n4, h.first, h.last);
+                    }
+                }
+            }
+            if (c.d_weight) {
+                const int tiles = v_tiles * h_tiles;
+                if (RLK_CHAIN_DW && H % 256 == 0 && tok_valid % kBK == 0 && tok_valid >= 2 * kBK)
+                    hipLaunchKernelGGL((linear_logp_dw_kernel<T, kBK, true>),
+                                       dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kChainSmem,
+                                       stream, d);
+                else
+                    hipLaunchKernelGGL((linear_logp_dw_kernel<T, kBK, false>), dim3(tiles),
+                                       dim3(kThreads), GW::kSmemBytes, stream, d);
+            }
+            if (c.d_bias != nullptr) {
+                hipLaunchKernelGGL(linear_logp_db_kernel, dim3((v_valid + 255) / 256), dim3(256), 0,
+                                   stream, dz, p.ldz, tok_valid, v_valid, scales, c.d_bias + v_lo,
+                                   ci > 0 ? 1 : 0, c.dtype);
+            }
+            if (int rc = check_launch("linear_logp backward launch failed")) return rc;
+        }
+    }
+    return 0;
 }
 
 int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const int64_t* targets,
@@ -1103,171 +1537,11 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                            workspace, N, H, V, vocab_start, dtype, temperature, ignore_index,
                            use_ignore, stream);
     const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
-
-    char* ws = static_cast<char*>(workspace);
-    float* scales = reinterpret_cast<float*>(ws + p.scales_off);
-    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.dz_off);
-    float* hacc = p.acc_bytes ? reinterpret_cast<float*>(ws + p.acc_off) : nullptr;
-    const uint16_t* hid = static_cast<const uint16_t*>(hidden);
-    const uint16_t* w = static_cast<const uint16_t*>(weight);
-    uint16_t* dh = static_cast<uint16_t*>(d_hidden);
-    const int h_tiles = (H + 255) / 256;
-
-    hipLaunchKernelGGL(linear_logp_scales_kernel, dim3(1), dim3(1024), 0, stream, grad_logp,
-                       static_cast<int>(N), 1.f / temperature, dtype, scales);
-    if (int rc = check_launch("scales kernel launch failed")) return rc;
-
-    using GZb = TileGemm<Bf16, false, false, kBK>;
-    using GHb = TileGemm<Bf16, true, false, kBK>;
-    using GWb = TileGemm<Bf16, true, true, kBK>;
-    if (dtype == RLK_DTYPE_BF16) {
-        if (int rc = set_smem(linear_logp_dz_kernel<Bf16, kBK, false>, GZb::kSmemBytes)) return rc;
-        if (int rc = set_smem(linear_logp_dz_kernel<Bf16, kBK, true>, GZb::kSmemBytes)) return rc;
-        if (int rc = set_smem(linear_logp_dh_kernel<Bf16, kBK>, GHb::kSmemBytes)) return rc;
-        if (int rc = set_smem(linear_logp_dw_kernel<Bf16, kBK>, GWb::kSmemBytes)) return rc;
-    } else {
-        if (int rc = set_smem(linear_logp_dz_kernel<F16, kBK, false>, GZb::kSmemBytes)) return rc;
-        if (int rc = set_smem(linear_logp_dz_kernel<F16, kBK, true>, GZb::kSmemBytes)) return rc;
-        if (int rc = set_smem(linear_logp_dh_kernel<F16, kBK>, GHb::kSmemBytes)) return rc;
-        if (int rc = set_smem(linear_logp_dw_kernel<F16, kBK>, GWb::kSmemBytes)) return rc;
-    }
-
-    for (int ci = 0; ci < p.n_chunks; ++ci) {
-        const int64_t tok_lo = static_cast<int64_t>(ci) * p.tok_chunk;
-        const int tok_valid = static_cast<int>((N - tok_lo) < p.tok_chunk ? (N - tok_lo) : p.tok_chunk);
-        if (tok_valid <= 0) break;
-        const int tok_tiles = (tok_valid + 255) / 256;
-        for (int pi = 0; pi < p.n_pieces; ++pi) {
-            const int64_t v_lo = static_cast<int64_t>(pi) * p.v_piece;
-            const int v_valid = static_cast<int>((V - v_lo) < p.v_piece ? (V - v_lo) : p.v_piece);
-            if (v_valid <= 0) break;
-            const int v_tiles = (v_valid + 255) / 256;
-            const bool last_piece = (v_lo + p.v_piece >= V);
-
-            DzArgs z;
-            z.hidden = hid + tok_lo * H;
-            z.weight = w + v_lo * H;
-            z.bias = bias ? bias + v_lo : nullptr;
-            z.targets = targets + tok_lo;
-            z.lse = lse + tok_lo;
-            z.grad = grad_logp + tok_lo;
-            z.scales = scales;
-            z.dz = dz;
-            z.ldz = p.v_piece;
-            z.tok_valid = tok_valid;
-            z.v_valid = v_valid;
-            z.H = H;
-            z.tok_tiles = tok_tiles;
-            z.v_global0 = vocab_start + v_lo;
-            z.ignore_index = ignore_index;
-            z.use_ignore = use_ignore;
-            z.scale2 = kLog2e / temperature;
-
-            DhArgs h;
-            h.dz = dz;
-            h.weight = w + v_lo * H;
-            h.scales = scales;
-            h.acc = hacc;
-            h.out = dh ? dh + tok_lo * H : nullptr;
-            h.ldz = p.v_piece;
-            h.H = H;
-            h.v_valid = v_valid;
-            h.tok_valid = tok_valid;
-            h.tok_tiles = tok_tiles;
-            h.h_tiles = h_tiles;
-            h.first = pi == 0;
-            h.last = last_piece;
-            h.ksplit = p.ksplit;
-            h.part = p.ksplit > 1 ? reinterpret_cast<float*>(ws + p.part_off) : nullptr;
-            h.part_stride = static_cast<int64_t>(p.tok_chunk) * H;
-
-            DwArgs d;
-            d.dz = dz;
-            d.hidden = hid + tok_lo * H;
-            d.scales = scales;
-            d.dw = d_weight ? d_weight + v_lo * H : nullptr;
-            d.ldz = p.v_piece;
-            d.H = H;
-            d.v_valid = v_valid;
-            d.tok_valid = tok_valid;
-            d.v_tiles = v_tiles;
-            d.h_tiles = h_tiles;
-            d.accumulate = ci > 0;
-
-            // dZ block: full vocab tiles through the fast variant, the rest (all of them when
-            // there is a bias) through the general one
-            const int fast_tiles = bias ? 0 : v_valid / 256;
-            const int gen_tiles = v_tiles - fast_tiles;
-            if (dtype == RLK_DTYPE_BF16) {
-                if (fast_tiles > 0) {
-                    z.v_tiles = fast_tiles;
-                    z.v_tile_lo = 0;
-                    hipLaunchKernelGGL((linear_logp_dz_kernel<Bf16, kBK, false>),
-                                       dim3(tok_tiles * fast_tiles), dim3(kThreads), GZb::kSmemBytes,
-                                       stream, z);
-                }
-                if (gen_tiles > 0) {
-                    z.v_tiles = gen_tiles;
-                    z.v_tile_lo = fast_tiles;
-                    hipLaunchKernelGGL((linear_logp_dz_kernel<Bf16, kBK, true>),
-                                       dim3(tok_tiles * gen_tiles), dim3(kThreads), GZb::kSmemBytes,
-                                       stream, z);
-                }
-                if (d_hidden) {
-                    hipLaunchKernelGGL((linear_logp_dh_kernel<Bf16, kBK>),
-                                       dim3(tok_tiles * h_tiles * p.ksplit), dim3(kThreads),
-                                       GHb::kSmemBytes, stream, h);
-                    if (p.ksplit > 1) {
-                        const int64_t n4 = static_cast<int64_t>(tok_valid) * H / 4;
-                        hipLaunchKernelGGL((linear_logp_dh_reduce_kernel<Bf16>),
-                                           dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0,
-                                           stream, h.part, p.ksplit, h.part_stride, h.acc, h.out,
-                                           scales, n4, h.first, h.last);
-                    }
-                }
-                if (d_weight)
-                    hipLaunchKernelGGL((linear_logp_dw_kernel<Bf16, kBK>), dim3(v_tiles * h_tiles),
-                                       dim3(kThreads), GWb::kSmemBytes, stream, d);
-            } else {
-                if (fast_tiles > 0) {
-                    z.v_tiles = fast_tiles;
-                    z.v_tile_lo = 0;
-                    hipLaunchKernelGGL((linear_logp_dz_kernel<F16, kBK, false>),
-                                       dim3(tok_tiles * fast_tiles), dim3(kThreads), GZb::kSmemBytes,
-                                       stream, z);
-                }
-                if (gen_tiles > 0) {
-                    z.v_tiles = gen_tiles;
-                    z.v_tile_lo = fast_tiles;
-                    hipLaunchKernelGGL((linear_logp_dz_kernel<F16, kBK, true>),
-                                       dim3(tok_tiles * gen_tiles), dim3(kThreads), GZb::kSmemBytes,
-                                       stream, z);
-                }
-                if (d_hidden) {
-                    hipLaunchKernelGGL((linear_logp_dh_kernel<F16, kBK>),
-                                       dim3(tok_tiles * h_tiles * p.ksplit), dim3(kThreads),
-                                       GHb::kSmemBytes, stream, h);
-                    if (p.ksplit > 1) {
-                        const int64_t n4 = static_cast<int64_t>(tok_valid) * H / 4;
-                        hipLaunchKernelGGL((linear_logp_dh_reduce_kernel<F16>),
-                                           dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0,
-                                           stream, h.part, p.ksplit, h.part_stride, h.acc, h.out,
-                                           scales, n4, h.first, h.last);
-                    }
-                }
-                if (d_weight)
-                    hipLaunchKernelGGL((linear_logp_dw_kernel<F16, kBK>), dim3(v_tiles * h_tiles),
-                                       dim3(kThreads), GWb::kSmemBytes, stream, d);
-            }
-            if (d_bias != nullptr) {
-                hipLaunchKernelGGL(linear_logp_db_kernel, dim3((v_valid + 255) / 256), dim3(256), 0,
-                                   stream, dz, static_cast<int64_t>(p.v_piece), tok_valid, v_valid,
-                                   scales, d_bias + v_lo, ci > 0 ? 1 : 0, dtype);
-            }
-            if (int rc = check_launch("linear_logp backward launch failed")) return rc;
-        }
-    }
-    return 0;
+    int n_cu = 0;
+    if (int rc = compute_units(&n_cu)) return rc;
+    BwdCall c{grad_logp, hidden, weight, bias, targets, lse, d_hidden, d_weight, d_bias, workspace,
+              N, H, V, vocab_start, dtype, temperature, ignore_index, use_ignore, stream};
+    return dtype == RLK_DTYPE_BF16 ? bwd_enqueue<Bf16>(c, p, n_cu) : bwd_enqueue<F16>(c, p, n_cu);
 }
 
 }  // extern "C"
