@@ -64,7 +64,7 @@ const char* rlk_last_error(void);
  *   use_ignore != 0: rows whose target == ignore_index get logp = 0 exactly
  *            (rl_engine/testing/reference_ops.py:33-45; rl_engine/executors/deepspeed_trainer.py:559-569,639-641)
  *   strict_targets != 0: a non-ignored target outside [vocab_start, vocab_start + V) stores 1 to
- *            *err_flag (device int32, caller zeroes it); the Python layer turns that into the
+ *            *err_flag (device int32, caller zeroes it; may be NULL when strict_targets == 0); the Python layer turns that into the
  *            reference's ValueError (rl_engine/kernels/ops/cuda/loss/linear_logp.py:352-358).
  *            With strict_targets == 0 such a row yields logp = -lse (z_t = 0), which is what a
  *            vocab-parallel shard must return (csrc/cuda/fused_linear_logp_sm90.cu:256-280).
@@ -112,7 +112,9 @@ int rlk_linear_logp_fwd_static(const void* hidden, const void* weight, const flo
  *   d_weight = dZ^T H    (f32, overwritten)
  *   d_bias   = sum_n dZ  (f32, only when bias != NULL)
  * dZ only ever exists as one (token chunk) x (vocab piece) block of at most `dz_budget_bytes`
- * (0 = default 256 MiB) inside `workspace`, so extra memory does not grow with N.
+ * (0 = default 256 MiB; values are clamped to [128 KiB, 2 GiB], the upper limit keeping every
+ * in-tile byte offset of the loaders within 32 bits) inside `workspace`, so extra memory does not
+ * grow with N.
  * `lse` must be the natural-log logsumexp over the FULL vocabulary (for a shard: after the
  * cross-shard merge).  Any of d_hidden / d_weight / d_bias may be NULL to skip that gradient
  * (d_bias requires bias).

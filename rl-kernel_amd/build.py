@@ -3,6 +3,7 @@
 from __future__ import annotations
 
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -15,7 +16,8 @@ LIB_PATH = os.path.join(LIB_DIR, "librlk_hip.so")
 SOURCES = ["rlk_core.hip", "rlk_linear_logp.hip", "rlk_logp_scan.hip", "rlk_grpo.hip",
            "rlk_generic.hip"]
 
-# Packed-fp32 VALU forms are switched off for every device function of this library.
+# Packed-fp32 VALU forms are switched off for every device function of this library (the host pass
+# of hipcc warns that it does not know the feature; build() checks the device code instead).
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -30,29 +32,47 @@ def hipcc() -> str:
     return exe
 
 
+def _check_no_packed_fp32(asm_path: str, src: str) -> None:
+    """The switch-off of the packed-fp32 VALU forms is a device-side target feature; the host pass
+    of hipcc does not know it and says so.  What counts is the device code: it must not contain
+    a packed fp32 add / mul / fma."""
+    bad = re.compile(r"\bv_pk_(add|mul|fma)_f32\b")
+    with open(asm_path) as fh:
+        hits = [line.strip() for line in fh if bad.search(line)]
+    if hits:
+        raise RuntimeError(f"{src}: device code contains packed fp32 instructions "
+                           f"({len(hits)}, first: {hits[0]}); the -packed-fp32-ops switch did not take effect")
+
+
 def build(verbose: bool = False, extra_flags=()) -> str:
-    """Compile every source and link the shared library. Always recompiles."""
+    """Compile every source and link the shared library. Always recompiles.  Every source is
+    also compiled to device assembly once more to verify that no packed-fp32 instruction was
+    generated."""
     os.makedirs(LIB_DIR, exist_ok=True)
     objs = []
     procs = []
     for src in SOURCES:
         path = os.path.join(CSRC, src)
         if not os.path.exists(path):
-            continue
+            raise RuntimeError(f"source file {path} is missing")
         obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
+        asm = os.path.join(LIB_DIR, src.replace(".hip", ".device.s"))
         cmd = [hipcc(), *HIPCC_FLAGS, *extra_flags, "-c", path, "-o", obj]
+        chk = [hipcc(), *HIPCC_FLAGS, *extra_flags, "--cuda-device-only", "-S", path, "-o", asm]
         if verbose:
             print(" ".join(cmd), flush=True)
-        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+        procs.append((src, None, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+        procs.append((src, asm, subprocess.Popen(chk, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
         objs.append(obj)
-    for src, proc in procs:
+    for src, asm, proc in procs:
         out = proc.communicate()[0].decode()
         if proc.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{out}")
-        if verbose:
-            kept = [l for l in out.splitlines() if "not a recognized feature" not in l]
-            if kept:
-                print("\n".join(kept))
+        if verbose and asm is None and out.strip():
+            print(out)
+        if asm is not None:
+            _check_no_packed_fp32(asm, src)
+            os.remove(asm)
     tmp = LIB_PATH + ".tmp"
     link = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
     res = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)

@@ -14,6 +14,10 @@
 #define RLK_DEFAULT_DZ_BUDGET (static_cast<size_t>(256) << 20)  // bytes of one dZ block
 #endif
 
+#ifndef RLK_MAX_DZ_BUDGET
+#define RLK_MAX_DZ_BUDGET (static_cast<size_t>(2) << 30)  // upper clamp of dz_budget_bytes
+#endif
+
 // Records `msg` as the calling thread's last error and returns `code` (always negative).
 int rlk_fail(int code, const char* msg);
 

@@ -938,6 +938,17 @@ FwdPlan fwd_plan(int64_t N, int64_t V, bool has_bias)
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// One dZ block is at least one 256 x 256 tile and at most RLK_MAX_DZ_BUDGET bytes: the tile
+// loaders address rows inside a tile with 32-bit byte offsets (256 rows x leading dimension), so
+// the leading dimension of the block must stay below 2^23 elements.
+inline size_t clamp_dz_budget(size_t budget)
+{
+    if (budget == 0) budget = RLK_DEFAULT_DZ_BUDGET;
+    if (budget < 131072) budget = 131072;
+    if (budget > RLK_MAX_DZ_BUDGET) budget = RLK_MAX_DZ_BUDGET;
+    return budget;
+}
+
 struct BwdPlan {
     int tok_chunk;   // tokens per chunk (multiple of 256)
     int v_piece;     // vocab rows per piece (multiple of 256)
@@ -1068,6 +1079,7 @@ int check_common(int64_t N, int32_t H, int64_t V, int dtype)
         return rlk_fail(RLK_ERR_UNSUPPORTED, "dtype must be RLK_DTYPE_BF16, RLK_DTYPE_F16 or RLK_DTYPE_F32");
     if (N <= 0 || H <= 0 || V <= 0) return rlk_fail(RLK_ERR_ARG, "N, H and V must be positive");
     if (N > 0x7fff0000LL || V > 0x7fff0000LL) return rlk_fail(RLK_ERR_ARG, "N or V too large");
+    if (H > (1 << 20)) return rlk_fail(RLK_ERR_UNSUPPORTED, "hidden size above 2^20");
     return 0;
 }
 
@@ -1394,8 +1406,9 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
 {
     if (int rc = check_common(N, H, V, dtype)) return rc;
     if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
-    if (!hidden || !weight || !targets || !logp || !lse || !err_flag)
-        return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (!hidden || !weight || !targets || !logp || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (strict_targets && !err_flag)
+        return rlk_fail(RLK_ERR_ARG, "strict_targets needs an err_flag to report through");
     if (!use_mfma(hidden, weight, H, dtype))
         return generic_fwd(hidden, weight, bias, targets, logp, lse, N, H, V, vocab_start, dtype,
                            temperature, ignore_index, use_ignore, strict_targets, err_flag, stream);
@@ -1489,8 +1502,7 @@ int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t
 {
     (void)dtype;
     if (!bytes || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad workspace query");
-    if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
-    if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
+    dz_budget_bytes = clamp_dz_budget(dz_budget_bytes);
     // large enough for either implementation (the choice also depends on pointer alignment)
     const size_t a = bwd_plan(N, H, V, dz_budget_bytes).total, b = generic_bwd_workspace(N, H, V);
     *bytes = a > b ? a : b;
@@ -1502,8 +1514,7 @@ int rlk_linear_logp_bwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype, siz
 {
     (void)dtype;
     if (!out5 || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad plan query");
-    if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
-    if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
+    dz_budget_bytes = clamp_dz_budget(dz_budget_bytes);
     const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
     out5[0] = p.tok_chunk;
     out5[1] = p.v_piece;
@@ -1525,8 +1536,7 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
     if (!grad_logp || !hidden || !weight || !targets || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
     if (!d_hidden && !d_weight && !d_bias) return rlk_fail(RLK_ERR_ARG, "no gradient requested");
     if (bias == nullptr && d_bias != nullptr) return rlk_fail(RLK_ERR_ARG, "d_bias given without bias");
-    if (dz_budget_bytes == 0) dz_budget_bytes = RLK_DEFAULT_DZ_BUDGET;
-    if (dz_budget_bytes < 131072) dz_budget_bytes = 131072;
+    dz_budget_bytes = clamp_dz_budget(dz_budget_bytes);
     size_t need = 0;
     rlk_linear_logp_bwd_workspace_bytes(N, H, V, dtype, dz_budget_bytes, &need);
     if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");

@@ -57,6 +57,27 @@ def hip_path_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     )
 
 
+_scalar_path_warned = False
+
+
+def _warn_if_scalar_path(hidden_2d: torch.Tensor, weight: torch.Tensor) -> None:
+    """The MFMA tiles take bf16/f16 with H % 8 == 0 and 16-byte aligned matrices; everything else
+    runs on scalar-FMA kernels that are meant for small correctness-sized problems.  Say so once
+    when a large problem ends up there."""
+    global _scalar_path_warned
+    if _scalar_path_warned:
+        return
+    n, h = hidden_2d.shape
+    on_mfma = (hidden_2d.dtype in (torch.bfloat16, torch.float16) and h % 8 == 0
+               and hidden_2d.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+    if not on_mfma and n * h * weight.size(0) > (1 << 33):
+        _scalar_path_warned = True
+        logger.warning(
+            "linear_logp: %s inputs with H=%d run on the scalar-FMA kernels (the MFMA path takes "
+            "bf16/f16, H %% 8 == 0, 16-byte aligned matrices); expect this %d x %d x %d problem "
+            "to be slow", str(hidden_2d.dtype), h, n, h, weight.size(0))
+
+
 def fused_linear_logp_forward(
     hidden_2d: torch.Tensor,
     weight: torch.Tensor,
@@ -81,6 +102,9 @@ def fused_linear_logp_forward(
     logp = torch.empty(n, device=dev, dtype=torch.float32)
     lse = torch.empty(n, device=dev, dtype=torch.float32)
     err = torch.zeros(1, device=dev, dtype=torch.int32)
+    if n == 0:  # nothing to launch
+        return logp, lse, err
+    _warn_if_scalar_path(hidden_2d, weight)
     need = _native.ctypes.c_size_t(0)
     dt = _DTYPES[hidden_2d.dtype]
     _native.check(lib.rlk_linear_logp_fwd_workspace_bytes(n, h, v, dt, _native.ctypes.byref(need)),

@@ -5,9 +5,9 @@ Same contract as the reference's ``kernel_registry`` (rl_engine/kernels/registry
 instantiates with no arguments, caches the instance by backend name, remembers failed backends,
 and raises ``RuntimeError`` when none works.  On ROCm the gfx950 HIP backends come first; the
 reference maintainer's equivalent change is one enum entry per op at the head of
-``_priority_map["rocm"]``.  This mirror registers only the ops of the fused linear-logprob path;
-when the reference package is importable its portable PyTorch ops are listed as later candidates,
-otherwise a missing backend is an error rather than a silent CPU path.
+``_priority_map["rocm"]``.  This mirror registers only the gfx950 HIP backends of the fused
+linear-logprob path: a HIP backend that fails to load or construct is an error here, never a
+silent switch to a portable implementation, and the CPU platform has no backend at all.
 """
 
 from __future__ import annotations
@@ -35,11 +35,6 @@ class OpBackend(Enum, metaclass=_KernelEnumMeta):
     ROCM_RATIO_KL = "rl_kernel_amd.ops.grpo.RocmRatioKLOp"
     ROCM_GRPO_LOSS = "rl_kernel_amd.ops.grpo.RocmGRPOLossOp"
     ROCM_GRPO_FROM_LOGP = "rl_kernel_amd.ops.grpo.RocmGRPOFromLogpOp"
-    # portable ops of the reference package, used only when that package is installed
-    PYTORCH_LINEAR_LOGP = "rl_engine.kernels.ops.pytorch.loss.linear_logp.NativeLinearLogpOp"
-    PYTORCH_NATIVE = "rl_engine.kernels.ops.pytorch.loss.logp.NativeLogpOp"
-    PYTORCH_RATIO_KL = "rl_engine.kernels.ops.pytorch.loss.ratio_kl.NativeRatioKLOp"
-    PYTORCH_GRPO_LOSS = "rl_engine.kernels.ops.pytorch.loss.grpo_loss.NativeGRPOLossOp"
 
 
 _LOGP_TYPES = ("logp", "logp_indexed", "logp_online", "logp_online_indexed")
@@ -50,20 +45,16 @@ class KernelRegistry:
         self._instance_cache: Dict[str, Any] = {}
         self._failed_backends: Set[str] = set()
         rocm = {
-            "linear_logp": [OpBackend.ROCM_FUSED_LINEAR_LOGP, OpBackend.PYTORCH_LINEAR_LOGP],
-            "ratio_kl": [OpBackend.ROCM_RATIO_KL, OpBackend.PYTORCH_RATIO_KL],
-            "grpo_loss": [OpBackend.ROCM_GRPO_LOSS, OpBackend.PYTORCH_GRPO_LOSS],
+            "linear_logp": [OpBackend.ROCM_FUSED_LINEAR_LOGP],
+            "ratio_kl": [OpBackend.ROCM_RATIO_KL],
+            "grpo_loss": [OpBackend.ROCM_GRPO_LOSS],
             "grpo_loss_from_logp": [OpBackend.ROCM_GRPO_FROM_LOGP],
         }
-        cpu = {
-            "linear_logp": [OpBackend.PYTORCH_LINEAR_LOGP],
-            "ratio_kl": [OpBackend.PYTORCH_RATIO_KL],
-            "grpo_loss": [OpBackend.PYTORCH_GRPO_LOSS],
-        }
         for name in _LOGP_TYPES:
-            rocm[name] = [OpBackend.ROCM_FUSED_LOGP, OpBackend.PYTORCH_NATIVE]
-            cpu[name] = [OpBackend.PYTORCH_NATIVE]
-        self._priority_map = {"rocm": rocm, "cpu": cpu}
+            rocm[name] = [OpBackend.ROCM_FUSED_LOGP]
+        # no CPU backends: every op type is known on the CPU platform and answers with the
+        # "No functional backend" error
+        self._priority_map = {"rocm": rocm, "cpu": {name: [] for name in rocm}}
         logger.info("KernelRegistry initialized for %s", device_ctx.device_type)
 
     def platform(self) -> str:

@@ -140,3 +140,21 @@ def test_header_is_plain_c(tmp_path):
                           "-I", os.path.join(ROOT, "include"), str(src)],
                          capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
+
+
+@pytest.mark.parametrize("n,h,v", [(32768, 4096, 128256), (300, 4096, 2_000_000),
+                                   (2_000_000, 4096, 256), (1 << 20, 8192, 1 << 20)])
+@pytest.mark.parametrize("budget", [4 << 30, 64 << 30])
+def test_backward_plan_keeps_in_tile_offsets_within_32_bits(native, n, h, v, budget):
+    """Budgets of 4 GiB and more are clamped to 2 GiB: the tile loaders address the rows of one
+    256-row tile with 32-bit byte offsets, so 256 x (leading dimension of the dZ block) x 2 bytes
+    has to stay below 2^32 whatever the caller asks for, also for few tokens x a huge vocabulary
+    and for many tokens x a tiny one."""
+    lib = native.load()
+    tok_chunk, v_piece, n_chunks, n_pieces, _ = _plan(lib, n, h, v, 0, budget)
+    assert tok_chunk * v_piece * 2 <= 2 << 30
+    assert 256 * v_piece * 2 < 2 ** 32
+    assert tok_chunk * n_chunks >= n and v_piece * n_pieces >= v
+    need = ctypes.c_size_t(0)
+    assert lib.rlk_linear_logp_bwd_workspace_bytes(n, h, v, 0, budget, ctypes.byref(need)) == 0
+    assert need.value <= (3 << 30) + (1 << 20)          # block + fp32 dH chunk <= 1.5 x 2 GiB
