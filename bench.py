@@ -6,14 +6,25 @@
 One step = one forward (logp, lse) + one backward (dH in the input dtype, dW fp32) of the fused
 LM-head log-prob over one synthetic batch at the Llama-3-8B head shape (32768 tokens, H=4096,
 V=128256, bf16), through the C-ABI library.  Inputs are resident in HBM before the timed region.
-Prints ONE JSON line (metric = tokens/s of the whole step) carrying a `roofline` object for the
-dominant kernel (the forward contraction, timed with HIP events on the launch stream) and a
-`cpu_baseline` object (the CPU oracle timed on a bounded token slice on the host cores).
+
+Prints ONE JSON line.  Besides the headline metric (tokens/s of the whole step) it carries
+  * `kernels`: the four contraction kernels of the step (forward, dZ recompute, dH, dW), each with
+    its average launch time from HIP events on the launch stream, flops per launch and fraction
+    of the dense bf16 MFMA peak; `roofline` is the entry of the kernel that takes the most time;
+  * `through_registry_op`: the same step driven through `kernel_registry.get_op("linear_logp")`
+    and autograd (adds the target-range check and the cast of dW to the weight dtype);
+  * `extra_workloads`: the other benchmark configurations (64k tokens at T=0.7, the Qwen3 head in
+    f16 with 1 % ignored positions, the GRPO step with its loss epilogue, the logits-fed scan) and
+    the shapes the reference publishes H100 latencies for, a few steps each;
+  * `cpu_baseline`: the CPU oracle (F.linear -> log_softmax -> gather in fp32, autograd backward)
+    timed on a 2048-token slice on the host cores.
 """
 
 from __future__ import annotations
 
 import argparse
+import glob
+import hashlib
 import json
 import os
 import sys
@@ -24,12 +35,17 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}  # MI355X dense MFMA, published
+PEAK_HBM_GBS = 8000.0
 
-# HBM bytes moved by ONE forward launch of the default workload, from two `rocprofv3 --pmc` runs of
-# this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
-# reads for the 1 GiB `--calibrate-copy` kernel (factors 2.000 and 1.000):
-# 2.000 * 24869400 KiB + 1.000 * 1536 KiB.  Other workloads report null.
-MEASURED_FWD_TRAFFIC_BYTES = {"llama3-8b-head": (2.0 * 24869400 + 1536) * 1024}
+# HBM-side bytes moved by ONE launch of each kernel at the default workload, from two
+# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled
+# by what the same counter reads for the 1 GiB `--calibrate-copy` kernel.  The figures belong to
+# the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
+MEASURED_TRAFFIC = {
+    "workload": "llama3-8b-head",
+    "kernel_source_sha16": "",
+    "bytes_per_launch": {},
+}
 
 WORKLOADS = {
     # BASELINE.json configs[1] shape; the metric is quoted on forward+backward at this shape
@@ -51,14 +67,37 @@ WORKLOADS = {
                   ignore_frac=0.0),
 }
 
+# linear_logp latencies the reference publishes (docs/operators/linear-logp.md:116-132 of the
+# reference: NVIDIA H100 80GB, bf16, N=4096, D=2048), in ms: forward, forward+backward
+REFERENCE_PUBLISHED_H100 = {
+    32768: {"fwd_ms": {"native": 1.79, "triton": 6.42, "sm90": 3.41},
+            "fwd_bwd_ms": {"native": 4.25, "triton": 15.86, "sm90": 12.69}},
+    50257: {"fwd_ms": {"native": 9.96, "triton": 9.82, "sm90": 4.88},
+            "fwd_bwd_ms": {"native": 23.29, "triton": 47.20, "sm90": 42.20}},
+    131072: {"fwd_ms": {"native": 7.28, "triton": 25.56, "sm90": 12.88},
+             "fwd_bwd_ms": {"native": 17.05, "triton": 117.62, "sm90": 104.97}},
+}
+
+
+def kernel_source_sha16() -> str:
+    m = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(ROOT, "rl-kernel_amd", "csrc", "*"))):
+        with open(path, "rb") as fh:
+            m.update(os.path.basename(path).encode())
+            m.update(fh.read())
+    return m.hexdigest()[:16]
+
 
 def make_inputs(torch, cfg, device, seed=1002):
     gen = torch.Generator(device=device).manual_seed(seed)
     dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float16
     n, h, v = cfg["tokens"], cfg["hidden"], cfg["vocab"]
-    hidden = torch.randn(n, h, device=device, dtype=torch.float32, generator=gen).to(dt)
+    hidden = torch.empty(n, h, device=device, dtype=dt)
+    step = 16384  # generate in slabs to bound the fp32 temporary
+    for n0 in range(0, n, step):
+        n1 = min(n, n0 + step)
+        hidden[n0:n1] = torch.randn(n1 - n0, h, device=device, dtype=torch.float32, generator=gen).to(dt)
     weight = torch.empty(v, h, device=device, dtype=dt)
-    step = 16384  # generate W in slabs to bound the fp32 temporary
     for v0 in range(0, v, step):
         v1 = min(v, v0 + step)
         weight[v0:v1] = (torch.randn(v1 - v0, h, device=device, dtype=torch.float32,
@@ -71,21 +110,23 @@ def make_inputs(torch, cfg, device, seed=1002):
     return hidden, weight, targets, grad
 
 
-def cpu_baseline(torch, cfg, slice_tokens, iters=3):
-    """Time the CPU oracle (fp32 linear + log_softmax + gather, closed-form backward) on a slice."""
+def cpu_baseline(torch, cfg, slice_tokens, iters=2):
+    """Time the CPU oracle on a token slice: fp32 F.linear -> log_softmax -> gather forward, torch
+    autograd backward (what the reference's CPU path does for a training step)."""
     from oracle import oracle as O
 
     gen = torch.Generator().manual_seed(7)
     h, v = cfg["hidden"], cfg["vocab"]
-    hidden = torch.randn(slice_tokens, h, generator=gen)
-    weight = torch.randn(v, h, generator=gen) * 0.02
+    hidden = torch.randn(slice_tokens, h, generator=gen).requires_grad_(True)
+    weight = (torch.randn(v, h, generator=gen) * 0.02).requires_grad_(True)
     targets = torch.randint(0, v, (slice_tokens,), generator=gen)
     grad = torch.randn(slice_tokens, generator=gen)
 
     def step():
-        O.linear_logp(hidden, weight, targets, temperature=cfg["temperature"])
-        O.linear_logp_backward(grad, hidden, weight, targets, temperature=cfg["temperature"],
-                               token_chunk=1024)
+        hidden.grad = None
+        weight.grad = None
+        logp = O.linear_logp(hidden, weight, targets, temperature=cfg["temperature"])
+        logp.backward(grad)
 
     step()  # warm-up
     times = []
@@ -94,15 +135,15 @@ def cpu_baseline(torch, cfg, slice_tokens, iters=3):
         step()
         times.append(time.perf_counter() - t0)
     times.sort()
-    med = times[len(times) // 2]
+    med = times[len(times) // 2] if len(times) % 2 else 0.5 * (times[len(times) // 2 - 1] + times[len(times) // 2])
     return {
         "value": slice_tokens / med,
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"{slice_tokens}-token slice at the full H={h}, V={v}; fp32 torch CPU oracle "
-                  f"forward+backward, 1 warm-up + {iters} timed, median; host cpu_count="
-                  f"{os.cpu_count()}",
+                  f"(F.linear -> log_softmax -> gather) forward + autograd backward, 1 warm-up + "
+                  f"{iters} timed, median; host cpu_count={os.cpu_count()}",
     }
 
 
@@ -116,7 +157,21 @@ def device_info(torch):
     return info
 
 
-def bench_scan(torch, args, cfg) -> int:
+def event_ms(torch, fn, reps):
+    """Average duration of fn() over `reps` back-to-back calls, by HIP events on the current
+    stream (the stream every kernel of this library is launched on)."""
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def bench_scan(torch, steps, warmup, cfg):
     """logp from materialised logits (rlk_logp_from_logits): one pass over N x V logits."""
     from rl_kernel_amd.ops.logp import logp_from_logits
 
@@ -130,84 +185,50 @@ def bench_scan(torch, args, cfg) -> int:
     ids = torch.randint(0, v, (n,), device=dev, generator=gen)
     out = torch.empty(n, device=dev, dtype=torch.float32)
     first = logp_from_logits(logits, ids, out).clone()
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         logp_from_logits(logits, ids, out)
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    e0.record()
-    for _ in range(args.steps):
-        logp_from_logits(logits, ids, out)
-    e1.record()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    k_ms = e0.elapsed_time(e1) / args.steps
+    k_ms = event_ms(torch, lambda: logp_from_logits(logits, ids, out), steps)
+    ms = (time.perf_counter() - t0) * 1e3 / steps
     nbytes = float(n * v * logits.element_size() + n * 8 + n * 4)
-    result = {
+    return {
         "metric": "logp from logits tokens/sec", "value": n / (ms * 1e-3), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"],
         "data": "synthetic",
         "config": {"workload": f"logits-scan: selected-token logp from {n} x {v} {cfg['dtype']} logits",
                    "tokens": n, "vocab": v},
         "bitwise_repeatable": bool(torch.equal(first, out)),
-        "device": device_info(torch),
         "roofline": {"kernel": "logp_scan_kernel", "bound": "hbm", "achieved": nbytes / (k_ms * 1e-3) / 1e9,
-                     "peak": 8000.0, "unit": "GB/s", "frac": nbytes / (k_ms * 1e-3) / 1e9 / 8000.0,
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": nbytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                      "traffic": None, "algorithmic_bytes": nbytes, "launch_ms": k_ms},
     }
-    print(json.dumps(result))
-    return 0
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="llama3-8b-head", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-slice", type=int, default=1024,
-                    help="tokens of the CPU-baseline slice (0 = skip the CPU baseline)")
-    ap.add_argument("--mode", default="fwd+bwd", choices=["fwd+bwd", "fwd"])
-    ap.add_argument("--dtype", default=None, choices=["bf16", "f16"],
-                    help="override the workload's 16-bit input type")
-    ap.add_argument("--no-library-gemm", action="store_true",
-                    help="skip the vendor-GEMM comparison figure")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one plain 1 GiB device copy (known HBM traffic) so that a "
-                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
-    args = ap.parse_args()
+def bwd_plan(n, h, v, dtype_id):
+    import ctypes
 
-    if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; every figure is a one-GPU figure. "
-              "Run with --gpus 1.", file=sys.stderr)
-        return 2
+    from rl_kernel_amd import _native
 
-    import torch
+    out = (ctypes.c_int64 * 5)()
+    _native.check(_native.load().rlk_linear_logp_bwd_plan(n, h, v, dtype_id, 0, out), "plan")
+    return dict(tok_chunk=out[0], v_piece=out[1], n_chunks=out[2], n_pieces=out[3], dh_parts=out[4])
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
-        return 3
 
+def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False):
+    """Forward(+backward) of the fused LM-head logp through the raw C-ABI wrappers."""
     from rl_kernel_amd.ops import linear_logp as LL
 
-    cfg = dict(WORKLOADS[args.workload])
-    if args.dtype:
-        cfg["dtype"] = args.dtype
-    if cfg.get("scan"):
-        return bench_scan(torch, args, cfg)
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
     hidden, weight, targets, grad = make_inputs(torch, cfg, dev)
     n, h, v = cfg["tokens"], cfg["hidden"], cfg["vocab"]
     ign = -100 if cfg["ignore_frac"] > 0 else None
     temp = cfg["temperature"]
-    do_bwd = args.mode == "fwd+bwd"
-
-    fwd_ev = []
-    epi_ev = []
+    do_bwd = mode == "fwd+bwd"
+    peak = PEAK_TFLOPS[cfg["dtype"]]
     grpo = cfg.get("grpo")
+    epi_ev = []
     if grpo:
         from rl_kernel_amd.ops import grpo as GR
 
@@ -224,42 +245,256 @@ def main() -> int:
         rewards = torch.randn(g, device=dev, generator=gen)
         del new_logp
 
-    def grpo_step(record):
-        logp, lse, _ = LL.fused_linear_logp_forward(hidden, weight, targets, None,
-                                                    temperature=temp, ignore_index=ign)
-        if record:
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
-            e0.record()
-        adv = GR.group_advantages(rewards, samples_per_prompt=g)
-        out3, _, _, d_cur, _ = GR.grpo_from_logp_raw(logp.view(g, t), old, ref, adv, mask,
-                                                     clip_eps=grpo["clip_eps"], beta=grpo["beta"],
-                                                     want_grad=True)
-        if record:
-            e1.record()
-            epi_ev.append((e0, e1))
-        d_h, d_w, _ = LL.fused_linear_logp_backward(d_cur.reshape(-1), hidden, weight, targets, lse,
-                                                    None, temperature=temp, ignore_index=ign)
-        return (logp, lse, out3, d_h, d_w)
+    def forward():
+        return LL.fused_linear_logp_forward(hidden, weight, targets, None, temperature=temp,
+                                            ignore_index=ign)
+
+    def backward(upstream, lse, need_hidden=True, need_weight=True):
+        return LL.fused_linear_logp_backward(upstream, hidden, weight, targets, lse, None,
+                                             temperature=temp, ignore_index=ign,
+                                             need_hidden=need_hidden, need_weight=need_weight)
 
     def step(record=False):
+        logp, lse, _ = forward()
+        if not do_bwd:
+            return (logp, lse)
+        upstream = grad
+        extra = ()
         if grpo:
-            return grpo_step(record)
-        if record:
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
-            e0.record()
-        logp, lse, err = LL.fused_linear_logp_forward(hidden, weight, targets, None,
-                                                      temperature=temp, ignore_index=ign)
-        if record:
-            e1.record()
-            fwd_ev.append((e0, e1))
-        out = (logp, lse)
-        if do_bwd:
-            d_h, d_w, _ = LL.fused_linear_logp_backward(grad, hidden, weight, targets, lse, None,
-                                                        temperature=temp, ignore_index=ign)
-            out = (logp, lse, d_h, d_w)
+            if record:
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+            adv = GR.group_advantages(rewards, samples_per_prompt=g)
+            out3, _, _, d_cur, _ = GR.grpo_from_logp_raw(logp.view(g, t), old, ref, adv, mask,
+                                                         clip_eps=grpo["clip_eps"], beta=grpo["beta"],
+                                                         want_grad=True)
+            if record:
+                e1.record()
+                epi_ev.append((e0, e1))
+            upstream = d_cur.reshape(-1)
+            extra = (out3,)
+        d_h, d_w, _ = backward(upstream, lse)
+        return (logp, lse) + extra + (d_h, d_w)
+
+    torch.cuda.synchronize()
+    base_mem = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    first = step()
+    torch.cuda.synchronize()
+    out_bytes = sum(t.numel() * t.element_size() for t in first)
+    peak_extra = torch.cuda.max_memory_allocated() - base_mem - out_bytes
+    for _ in range(max(0, warmup - 1)):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    last = None
+    for _ in range(steps):
+        last = step(record=True)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    deterministic = all(torch.equal(a, b) for a, b in zip(first, last))
+    lse = last[1]
+    del first, last
+
+    step_flops = (8.0 if do_bwd else 2.0) * n * h * v
+    res = {
+        "metric": "logp fwd+bwd tokens/sec" if do_bwd else "logp fwd tokens/sec",
+        "value": n / (ms * 1e-3),
+        "unit": "tokens/s",
+        "ms_per_step": ms,
+        "dtype": cfg["dtype"],
+        "config": {
+            "workload": f"{name}: fused LM-head logp {mode}, {n} tokens, H={h}, "
+                        f"V={v}, {cfg['dtype']} in / fp32 accumulate, T={temp}",
+            "tokens": n, "hidden": h, "vocab": v, "mode": mode,
+        },
+        "step_tflops": step_flops / (ms * 1e-3) / 1e12,
+        "step_frac_of_mfma_peak": step_flops / (ms * 1e-3) / 1e12 / peak,
+        "step_flop_accounting": "8*N*H*V (fwd 2 + logit recompute 2 + dH 2 + dW 2)" if do_bwd
+                                else "2*N*H*V",
+        "step_tflops_no_recompute_accounting": (6.0 if do_bwd else 2.0) * n * h * v / (ms * 1e-3) / 1e12,
+        "peak_extra_hbm_bytes": int(peak_extra),
+        "peak_extra_hbm_note": "raw C ABI: logp, lse, dH and the fp32 dW are declared outputs; what "
+                               "is counted is workspace (split partials, one dZ block, fp32 dH chunk)",
+        "bitwise_repeatable": bool(deterministic),
+    }
+    if grpo:
+        epi_ms = sum(a.elapsed_time(b) for a, b in epi_ev) / len(epi_ev)
+        epi_bytes = n * (4 + 4 + 4 + 1 + 4 + 4)  # cur, old, ref, mask in; d_cur, d_kl out
+        res["metric"] = "GRPO step (logp fwd + loss epilogue + bwd) tokens/sec"
+        res["epilogue"] = {
+            "bound": "hbm", "ms": epi_ms, "algorithmic_bytes": epi_bytes,
+            "achieved": epi_bytes / (epi_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": epi_bytes / (epi_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+            "note": "group advantages + loss/grad launches incl. host launch gaps; 0.7 MB of "
+                    "traffic, launch-latency-bound",
+            "active_tokens": int(mask.sum().item()),
+        }
+
+    # per-kernel launch times by HIP events: the forward on its own; the three backward kernels
+    # from backward calls with one gradient switched off (dZ+dH, dZ+dW, all three), by difference
+    reps = 3 if detailed else 2
+    fwd_ms = event_ms(torch, forward, reps)
+    fwd_flops = 2.0 * n * h * v
+    kernels = [{"kernel": "linear_logp_fwd_kernel", "launches_per_step": 1, "launch_ms": fwd_ms,
+                "flops_per_launch": fwd_flops, "achieved": fwd_flops / (fwd_ms * 1e-3) / 1e12,
+                "algorithmic_bytes": float((n * h + v * h) * 2 + n * 8 + n * 8)}]
+    if do_bwd and detailed:
+        plan = bwd_plan(n, h, v, 0 if cfg["dtype"] == "bf16" else 1)
+        blocks = plan["n_chunks"] * plan["n_pieces"]
+        t_all = event_ms(torch, lambda: backward(grad, lse), reps)
+        t_h = event_ms(torch, lambda: backward(grad, lse, need_weight=False), reps)
+        t_w = event_ms(torch, lambda: backward(grad, lse, need_hidden=False), reps)
+        blk_flops = 2.0 * n * h * v / blocks
+        elt = 2
+        c, p = min(plan["tok_chunk"], n), min(plan["v_piece"], v)
+        alg = {"linear_logp_dz_kernel": (c * h + p * h + c * p) * elt,
+               "linear_logp_dh_kernel": (c * p + p * h) * elt + c * h * 4,
+               "linear_logp_dw_kernel": (c * p + c * h) * elt + p * h * 4}
+        for kname, total in (("linear_logp_dz_kernel", t_h + t_w - t_all),
+                             ("linear_logp_dh_kernel", t_all - t_w),
+                             ("linear_logp_dw_kernel", t_all - t_h)):
+            kernels.append({"kernel": kname, "launches_per_step": blocks,
+                            "launch_ms": total / blocks, "flops_per_launch": blk_flops,
+                            "achieved": blk_flops / (total / blocks * 1e-3) / 1e12,
+                            "algorithmic_bytes": float(alg[kname])})
+        res["backward_plan"] = plan
+        res["backward_ms"] = t_all
+        res["kernel_timing_method"] = (
+            "HIP events on the launch stream; forward alone; backward kernels from three backward "
+            "calls (all gradients, without dW, without dH) by difference, divided by the number of "
+            "(token chunk x vocab piece) blocks")
+    sha = kernel_source_sha16()
+    for k in kernels:
+        k.update({"bound": "mfma", "peak": peak, "unit": "TFLOP/s", "frac": k["achieved"] / peak})
+        traffic = None
+        if name == MEASURED_TRAFFIC["workload"] and sha == MEASURED_TRAFFIC["kernel_source_sha16"]:
+            traffic = MEASURED_TRAFFIC["bytes_per_launch"].get(k["kernel"])
+        k["traffic"] = traffic
+    res["kernels"] = kernels
+    res["kernel_source_sha16"] = sha
+    dominant = max(kernels, key=lambda k: k["launch_ms"] * k["launches_per_step"])
+    res["roofline"] = dict(dominant)
+    res["roofline"]["note"] = "the kernel with the largest share of the step; see `kernels` for all four"
+
+    if detailed and do_bwd and not grpo:
+        res["through_registry_op"] = bench_registry_op(torch, hidden, weight, targets, grad, temp, ign,
+                                                       max(2, steps // 4))
+    return res
+
+
+def bench_registry_op(torch, hidden, weight, targets, grad, temp, ign, steps):
+    """The same step through kernel_registry.get_op('linear_logp') and autograd."""
+    from rl_kernel_amd.registry import kernel_registry
+
+    op = kernel_registry.get_op("linear_logp")
+    hid = hidden.detach().requires_grad_(True)
+    w = weight.detach().requires_grad_(True)
+
+    def step():
+        hid.grad = None
+        w.grad = None
+        out = op(hid, w, targets, temperature=temp, ignore_index=ign)
+        out.backward(grad)
         return out
+
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    out = step()
+    torch.cuda.synchronize()
+    declared = out.numel() * 4 + hid.grad.numel() * hid.grad.element_size() + \
+        w.grad.numel() * w.grad.element_size()
+    peak_extra = torch.cuda.max_memory_allocated() - base - declared
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    n = hidden.size(0)
+    return {"class": type(op).__name__, "ms_per_step": ms, "tokens_per_s": n / (ms * 1e-3),
+            "steps": steps, "peak_extra_hbm_bytes": int(peak_extra),
+            "note": "declared outputs here are logp, dH and dW in the weight dtype; the extra bytes "
+                    "include the fp32 dW the kernels accumulate into before the cast (as the "
+                    "reference's backward keeps an fp32 grad_w) and the saved lse"}
+
+
+def bench_reference_shapes(torch):
+    """The reference's own benchmark shapes and method (benchmarks/benchmark_linear_logp.py:62-86:
+    bf16, hidden ~ N(0,1), weight ~ N(0,1), warm-up 5, 20 iterations between device events),
+    through the op class and autograd, next to the H100 latencies the reference publishes."""
+    from rl_kernel_amd.registry import kernel_registry
+
+    op = kernel_registry.get_op("linear_logp")
+    dev = torch.device("cuda:0")
+    rows = []
+    for vocab, published in REFERENCE_PUBLISHED_H100.items():
+        n, d = 4096, 2048
+        gen = torch.Generator(device=dev).manual_seed(vocab)
+        hidden = torch.randn(n, d, device=dev, generator=gen).to(torch.bfloat16).requires_grad_(True)
+        weight = torch.randn(vocab, d, device=dev, generator=gen).to(torch.bfloat16).requires_grad_(True)
+        target = torch.randint(0, vocab, (n,), device=dev, generator=gen)
+
+        def fwd():
+            with torch.no_grad():
+                return op(hidden, weight, target)
+
+        def fwd_bwd():
+            hidden.grad = None
+            weight.grad = None
+            op(hidden, weight, target).sum().backward()
+
+        for _ in range(5):
+            fwd()
+            fwd_bwd()
+        rows.append({"shape": f"{n}x{d}x{vocab}", "fwd_ms": event_ms(torch, fwd, 20),
+                     "fwd_bwd_ms": event_ms(torch, fwd_bwd, 20),
+                     "reference_h100_ms": published})
+        del hidden, weight
+    return {"what": "linear_logp latency at the shapes of the reference's published table, op class + "
+                    "autograd on one MI355X; reference_h100_ms are the reference's own H100 figures "
+                    "(other hardware: context, not a like-for-like baseline)",
+            "rows": rows}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama3-8b-head", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-slice", type=int, default=2048,
+                    help="tokens of the CPU-baseline slice (0 = skip the CPU baseline)")
+    ap.add_argument("--mode", default="fwd+bwd", choices=["fwd+bwd", "fwd"])
+    ap.add_argument("--dtype", default=None, choices=["bf16", "f16"],
+                    help="override the workload's 16-bit input type")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the extra workloads, the registry-op timing and the vendor GEMM")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (known HBM traffic) so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; every figure is a one-GPU figure. "
+              "Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
+        return 3
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = dict(WORKLOADS[args.workload])
+    if args.dtype:
+        cfg["dtype"] = args.dtype
+    common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
+              "scaling": "weak", "vs_baseline": None, "data": "synthetic", "seed": 1002}
 
     if args.calibrate_copy:
         src = torch.ones(1 << 28, device=dev, dtype=torch.float32)   # 1 GiB read + 1 GiB written
@@ -268,114 +503,57 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
-    torch.cuda.synchronize()
-    base_mem = torch.cuda.memory_allocated()
-    torch.cuda.reset_peak_memory_stats()
-    first = step()
-    torch.cuda.synchronize()
-    out_bytes = sum(t.numel() * t.element_size() for t in first)
-    peak_extra = torch.cuda.max_memory_allocated() - base_mem - out_bytes
-    for _ in range(max(0, args.warmup - 1)):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    last = None
-    for _ in range(args.steps):
-        last = step(record=True)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms = elapsed * 1e3 / args.steps
 
-    deterministic = all(torch.equal(a, b) for a, b in zip(first, last))
-    if grpo:
-        # the forward launch is timed on its own after the steps (the step brackets the epilogue)
-        for _ in range(3):
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
-            e0.record()
-            LL.fused_linear_logp_forward(hidden, weight, targets, None, temperature=temp,
-                                         ignore_index=ign)
-            e1.record()
-            fwd_ev.append((e0, e1))
-        torch.cuda.synchronize()
-    fwd_ms = sum(a.elapsed_time(b) for a, b in fwd_ev) / len(fwd_ev)
-    fwd_flops = 2.0 * n * h * v
-    achieved = fwd_flops / (fwd_ms * 1e-3) / 1e12
-    peak = PEAK_TFLOPS[cfg["dtype"]]
-    step_flops = (8.0 if do_bwd else 2.0) * n * h * v
+    if cfg.get("scan"):
+        result = bench_scan(torch, args.steps, args.warmup, cfg)
+        result["device"] = device_info(torch)
+        print(json.dumps(result))
+        return 0
 
-    result = {
-        "metric": "logp fwd+bwd tokens/sec" if do_bwd else "logp fwd tokens/sec",
-        "value": n / (ms * 1e-3),
-        "unit": "tokens/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": cfg["dtype"],
-        "data": "synthetic",
-        "config": {
-            "workload": f"{args.workload}: fused LM-head logp {args.mode}, {n} tokens, H={h}, "
-                        f"V={v}, {cfg['dtype']} in / fp32 accumulate, T={temp}",
-            "tokens": n, "hidden": h, "vocab": v, "mode": args.mode,
-        },
-        "step_tflops": step_flops / (ms * 1e-3) / 1e12,
-        "step_frac_of_mfma_peak": step_flops / (ms * 1e-3) / 1e12 / peak,
-        "step_flop_accounting": "8*N*H*V (fwd 2 + logit recompute 2 + dH 2 + dW 2)" if do_bwd
-                                else "2*N*H*V",
-        "step_tflops_no_recompute_accounting": (6.0 if do_bwd else 2.0) * n * h * v / (ms * 1e-3) / 1e12,
-        "peak_extra_hbm_bytes": int(peak_extra),
-        "device": device_info(torch),
-        "seed": 1002,
-        "bitwise_repeatable": bool(deterministic),
-        "roofline": {
-            "kernel": "linear_logp_fwd_kernel",
-            "bound": "mfma",
-            "achieved": achieved,
-            "peak": peak,
-            "unit": "TFLOP/s",
-            "frac": achieved / peak,
-            "traffic": MEASURED_FWD_TRAFFIC_BYTES.get(args.workload),
-            "algorithmic_bytes": float((n * h + v * h) * 2 + n * 8 + n * 8),
-            "launch_ms": fwd_ms,
-            "flops_per_launch": fwd_flops,
-        },
-    }
-    if not args.no_library_gemm:
-        # vendor GEMM (torch.matmul -> hipBLASLt) on the same box at the same H, for scale only:
-        # hidden [N, H] x W[:16384]^T -> [N, 16384] in the input dtype
+    main_default = args.workload == "llama3-8b-head" and args.mode == "fwd+bwd" and not args.no_extras
+    result = dict(common)
+    result.update(bench_linear(torch, args.workload, cfg, args.steps, args.warmup, args.mode,
+                               detailed=not args.no_extras))
+    result["device"] = device_info(torch)
+    torch.cuda.empty_cache()
+
+    if not args.no_extras:
+        # vendor GEMM (torch.matmul -> hipBLASLt) on the same box at the same H, for scale only
         try:
-            wv = weight[: min(v, 16384)]
-            torch.matmul(hidden, wv.t())
-            torch.cuda.synchronize()
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(5):
-                torch.matmul(hidden, wv.t())
-            e1.record()
-            torch.cuda.synchronize()
-            lib_ms = e0.elapsed_time(e1) / 5
+            n, h, v = cfg["tokens"], cfg["hidden"], cfg["vocab"]
+            dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float16
+            a = torch.randn(n, h, device=dev).to(dt)
+            b = (torch.randn(min(v, 16384), h, device=dev) * 0.02).to(dt)
+            torch.matmul(a, b.t())
+            lib_ms = event_ms(torch, lambda: torch.matmul(a, b.t()), 5)
             result["library_gemm"] = {
-                "what": f"torch.matmul [{n},{h}] x [{h},{wv.shape[0]}] {cfg['dtype']} (writes the logits it computes)",
-                "tflops": 2.0 * n * h * wv.shape[0] / (lib_ms * 1e-3) / 1e12, "ms": lib_ms}
+                "what": f"torch.matmul [{n},{h}] x [{h},{b.shape[0]}] {cfg['dtype']} (writes the logits it computes)",
+                "tflops": 2.0 * n * h * b.shape[0] / (lib_ms * 1e-3) / 1e12, "ms": lib_ms}
+            del a, b
         except Exception as exc:  # the comparison is optional
             result["library_gemm"] = {"error": str(exc)[:200]}
-    if grpo:
-        epi_ms = sum(a.elapsed_time(b) for a, b in epi_ev) / len(epi_ev)
-        epi_bytes = n * (4 + 4 + 4 + 1 + 4 + 4)  # cur, old, ref, mask in; d_cur, d_kl out
-        result["metric"] = "GRPO step (logp fwd + loss epilogue + bwd) tokens/sec"
-        result["epilogue"] = {
-            "bound": "hbm", "ms": epi_ms, "algorithmic_bytes": epi_bytes,
-            "achieved": epi_bytes / (epi_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
-            "frac": epi_bytes / (epi_ms * 1e-3) / 1e9 / 8000.0,
-            "note": "group advantages + loss/grad launches incl. host launch gaps; 0.7 MB of "
-                    "traffic, launch-latency-bound",
-            "active_tokens": int(mask.sum().item()),
-        }
+        torch.cuda.empty_cache()
+
+    if main_default:
+        extras = {}
+        for name in ("llama3-8b-head-64k", "qwen3-head", "llama3-8b-grpo-step"):
+            r = bench_linear(torch, name, dict(WORKLOADS[name]), 3, 1, "fwd+bwd", detailed=False)
+            keep = ("metric", "value", "unit", "ms_per_step", "dtype", "config", "step_tflops",
+                    "step_frac_of_mfma_peak", "peak_extra_hbm_bytes", "bitwise_repeatable",
+                    "epilogue")
+            extras[name] = {k: r[k] for k in keep if k in r}
+            extras[name]["forward_launch_ms"] = r["kernels"][0]["launch_ms"]
+            extras[name]["forward_tflops"] = r["kernels"][0]["achieved"]
+            extras[name]["steps"] = 3
+            torch.cuda.empty_cache()
+        r = bench_scan(torch, 10, 2, dict(WORKLOADS["logits-scan"]))
+        extras["logits-scan"] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "config",
+                                                   "bitwise_repeatable", "roofline")}
+        torch.cuda.empty_cache()
+        extras["reference-published-shapes"] = bench_reference_shapes(torch)
+        torch.cuda.empty_cache()
+        result["extra_workloads"] = extras
+
     if args.cpu_slice > 0:
         result["cpu_baseline"] = cpu_baseline(torch, cfg, args.cpu_slice)
     print(json.dumps(result))
