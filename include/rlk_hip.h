@@ -189,6 +189,29 @@ int rlk_grpo_loss_from_logp(const float* cur_logp, const float* old_logp, const 
                             const float* upstream, void* workspace, size_t workspace_bytes,
                             rlk_stream_t stream);
 
+/* Forward of the fused linear log-prob with the loss epilogue above folded into its last launch
+ * (the composition the trainer runs as two steps, rl_engine/executors/deepspeed_trainer.py:
+ * 146-167): logp / lse exactly as rlk_linear_logp_fwd, and out3 / ratio / kl_terms / d_cur / d_kl
+ * exactly as rlk_grpo_loss_from_logp(cur_logp = logp, upstream = NULL) -- same expressions, same
+ * reduction tree, same bits -- without a second pass over the tokens: the active-token count is
+ * taken from the mask before the contraction starts, the per-token terms and gradients leave the
+ * launch that merges the vocab splits, and the workgroup of that launch that finishes last (an
+ * integer ticket; the sums themselves use no atomics) adds up the block partials in block order.
+ * Workspace: rlk_linear_logp_fwd_grpo_workspace_bytes (16-byte aligned).  Bit-equality of the
+ * sums with the two-step route holds below 2^24 tokens. */
+int rlk_linear_logp_fwd_grpo_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                                             size_t* bytes);
+
+int rlk_linear_logp_fwd_grpo(const void* hidden, const void* weight, const float* bias,
+                             const int64_t* targets, float* logp, float* lse, void* workspace,
+                             size_t workspace_bytes, int64_t N, int32_t H, int64_t V,
+                             int64_t vocab_start, int32_t dtype, float temperature,
+                             int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
+                             int32_t* err_flag, const float* old_logp, const float* ref_logp,
+                             const float* advantages, int32_t adv_per_token, const uint8_t* mask,
+                             int64_t seq_len, float clip_eps, float beta, float* out3, float* ratio,
+                             float* kl_terms, float* d_cur, float* d_kl, rlk_stream_t stream);
+
 /* Per-group reward normalisation (x - mean_g) / sqrt(max(E_g[x^2] - mean_g^2, eps^2)) over CSR
  * group boundaries (int64 [num_groups + 1], device).  Stands in for
  * NativeGRPOLossOp.group_advantages (rl_engine/kernels/ops/pytorch/loss/grpo_loss.py:53-84) and

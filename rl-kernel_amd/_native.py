@@ -32,6 +32,12 @@ SIGNATURES = {
     "rlk_grpo_loss_workspace_bytes": (_c.c_int, [_i64, _c.POINTER(_sz)]),
     "rlk_grpo_loss_from_logp": (_c.c_int, [_vp, _vp, _vp, _vp, _i32, _vp, _i64, _i64, _f32, _f32,
                                            _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "rlk_linear_logp_fwd_grpo_workspace_bytes": (_c.c_int, [_i64, _i32, _i64, _i32,
+                                                            _c.POINTER(_sz)]),
+    "rlk_linear_logp_fwd_grpo": (_c.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i32, _i64,
+                                            _i64, _i32, _f32, _i64, _i32, _i32, _vp,
+                                            _vp, _vp, _vp, _i32, _vp, _i64, _f32, _f32, _vp, _vp,
+                                            _vp, _vp, _vp, _vp]),
     "rlk_group_advantages": (_c.c_int, [_vp, _vp, _i64, _f32, _vp, _vp]),
     "rlk_selftest_transpose_read": (_c.c_int, [_vp, _vp]),
 }

@@ -1,70 +1,9 @@
 // Log-prob-fed GRPO / PPO loss epilogue: per-token policy ratio, clipped surrogate and k3 KL,
 // masked token-mean with a fixed two-level reduction tree, and dloss/dlogp.  Also the per-group
 // reward normalisation.  All sums run in a fixed order (no atomics): same input, same bits.
-#include "rlk_common.hpp"
+#include "rlk_grpo.hpp"
 
 namespace rlk {
-
-constexpr int kRedThreads = 256;
-constexpr int kMaxBlocks = 1024;
-
-struct GrpoArgs {
-    const float* cur;
-    const float* old_lp;
-    const float* ref_lp;   // may be null: KL term is 0
-    const float* adv;      // per token [n] or per sequence [n / seq_len]
-    const uint8_t* mask;   // may be null: every token active
-    float* ratio;          // optional per-token outputs (masked entries 0)
-    float* kl_terms;
-    float* partial;        // [blocks][3]: policy sum, kl sum, active count
-    float* out3;           // loss, policy_loss, kl
-    float* denom;          // max(count, 1e-8) kept for the gradient kernel
-    float* dcur;
-    float* dkl;            // optional: d kl / d cur alone (not scaled by beta or upstream)
-    const float* upstream; // optional device scalar multiplying dcur
-    int64_t n;
-    int64_t seq_len;
-    int adv_per_token;
-    float clip_lo, clip_hi, beta;
-    int blocks;
-};
-
-struct Term {
-    float pol, kl, act;
-};
-
-__device__ inline float adv_of(const GrpoArgs& a, int64_t i)
-{
-    return a.adv_per_token ? a.adv[i] : a.adv[i / a.seq_len];
-}
-
-// Fixed tree: lanes of a wavefront (shuffle), then wavefronts through LDS, left to right.
-__device__ inline Term block_sum(Term t)
-{
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        t.pol += __shfl_down(t.pol, o);
-        t.kl += __shfl_down(t.kl, o);
-        t.act += __shfl_down(t.act, o);
-    }
-    __shared__ float sh[kRedThreads / 64][3];
-    if ((threadIdx.x & 63) == 0) {
-        sh[threadIdx.x >> 6][0] = t.pol;
-        sh[threadIdx.x >> 6][1] = t.kl;
-        sh[threadIdx.x >> 6][2] = t.act;
-    }
-    __syncthreads();
-    Term r{0.f, 0.f, 0.f};
-    if (threadIdx.x == 0) {
-#pragma unroll
-        for (int w = 0; w < kRedThreads / 64; ++w) {
-            r.pol += sh[w][0];
-            r.kl += sh[w][1];
-            r.act += sh[w][2];
-        }
-    }
-    return r;
-}
 
 // Block b owns the contiguous element range [b*per, (b+1)*per); thread t walks it with stride
 // 256 in ascending order.
@@ -78,16 +17,10 @@ __global__ __launch_bounds__(kRedThreads) void grpo_terms_kernel(GrpoArgs a)
         const bool on = a.mask == nullptr || a.mask[i] != 0;
         float r = 0.f, k = 0.f;
         if (on) {
-            const float c = a.cur[i];
-            r = expf(c - a.old_lp[i]);
-            const float ad = adv_of(a, i);
-            const float rc = fminf(fmaxf(r, a.clip_lo), a.clip_hi);
-            t.pol += -fminf(r * ad, rc * ad);
-            if (a.ref_lp != nullptr) {
-                const float d = a.ref_lp[i] - c;
-                k = expf(d) - d - 1.f;
-                t.kl += k;
-            }
+            float pol;
+            token_terms(a, i, a.cur[i], r, pol, k);
+            t.pol += pol;
+            if (a.ref_lp != nullptr) t.kl += k;
             t.act += 1.f;
         }
         if (a.ratio) a.ratio[i] = r;
@@ -101,45 +34,13 @@ __global__ __launch_bounds__(kRedThreads) void grpo_terms_kernel(GrpoArgs a)
     }
 }
 
-__global__ __launch_bounds__(kRedThreads) void grpo_finish_kernel(GrpoArgs a)
-{
-    Term t{0.f, 0.f, 0.f};
-    for (int b = threadIdx.x; b < a.blocks; b += kRedThreads) {
-        t.pol += a.partial[b * 3 + 0];
-        t.kl += a.partial[b * 3 + 1];
-        t.act += a.partial[b * 3 + 2];
-    }
-    const Term s = block_sum(t);
-    if (threadIdx.x == 0) {
-        const float denom = fmaxf(s.act, 1e-8f);
-        const float pol = s.pol / denom, kl = s.kl / denom;
-        a.out3[0] = pol + a.beta * kl;
-        a.out3[1] = pol;
-        a.out3[2] = kl;
-        a.denom[0] = denom;
-    }
-}
-
-// d loss / d cur.  torch semantics of the composition: `minimum` sends the gradient to the
-// smaller branch and splits it on ties; `clamp` passes it on the closed interval.
+// d loss / d cur of every token (needs the denominator the finish kernel left).
 __global__ void grpo_grad_kernel(GrpoArgs a)
 {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= a.n) return;
     float g = 0.f, gk = 0.f;
-    if (a.mask == nullptr || a.mask[i] != 0) {
-        const float c = a.cur[i];
-        const float r = expf(c - a.old_lp[i]);
-        const float ad = adv_of(a, i);
-        const float rc = fminf(fmaxf(r, a.clip_lo), a.clip_hi);
-        const float un = r * ad, cl = rc * ad;
-        const float inside = (r >= a.clip_lo && r <= a.clip_hi) ? 1.f : 0.f;
-        const float w_un = un < cl ? 1.f : (un == cl ? 0.5f : 0.f);
-        g = -(w_un * ad * r + (1.f - w_un) * ad * r * inside);
-        if (a.ref_lp != nullptr) gk = (1.f - expf(a.ref_lp[i] - c)) / a.denom[0];
-        g = g / a.denom[0] + a.beta * gk;
-        if (a.upstream != nullptr) g *= a.upstream[0];
-    }
+    if (a.mask == nullptr || a.mask[i] != 0) token_grad(a, i, a.cur[i], a.denom[0], g, gk);
     a.dcur[i] = g;
     if (a.dkl != nullptr) a.dkl[i] = gk;
 }
@@ -179,7 +80,7 @@ extern "C" {
 int rlk_grpo_loss_workspace_bytes(int64_t n_tokens, size_t* bytes)
 {
     if (!bytes || n_tokens < 0) return rlk_fail(RLK_ERR_ARG, "bad workspace query");
-    *bytes = (static_cast<size_t>(kMaxBlocks) * 3 + 4) * sizeof(float);
+    *bytes = (static_cast<size_t>(kMaxBlocks) * 3 + kGrpoTailFloats) * sizeof(float);
     return 0;
 }
 
@@ -207,6 +108,7 @@ int rlk_grpo_loss_from_logp(const float* cur_logp, const float* old_logp, const 
     a.kl_terms = kl_terms;
     a.partial = static_cast<float*>(workspace);
     a.denom = a.partial + kMaxBlocks * 3;
+    a.words = reinterpret_cast<int*>(a.denom + 4);
     a.out3 = out3;
     a.dcur = d_cur;
     a.dkl = d_kl;
@@ -218,12 +120,9 @@ int rlk_grpo_loss_from_logp(const float* cur_logp, const float* old_logp, const 
     a.clip_lo = 1.f - clip_eps;
     a.clip_hi = 1.f + clip_eps;
     a.beta = beta;
-    int64_t blocks = (n_tokens + 4095) / 4096;  // ~16 elements per thread
-    if (blocks < 1) blocks = 1;
-    if (blocks > kMaxBlocks) blocks = kMaxBlocks;
-    a.blocks = static_cast<int>(blocks);
+    a.blocks = grpo_blocks(n_tokens);
     hipLaunchKernelGGL(grpo_terms_kernel, dim3(a.blocks), dim3(kRedThreads), 0, stream, a);
-    hipLaunchKernelGGL(grpo_finish_kernel, dim3(1), dim3(kRedThreads), 0, stream, a);
+    hipLaunchKernelGGL(grpo_finish_kernel<0>, dim3(1), dim3(kRedThreads), 0, stream, a);
     if (d_cur != nullptr && n_tokens > 0)
         hipLaunchKernelGGL(grpo_grad_kernel, dim3(static_cast<unsigned>((n_tokens + 255) / 256)),
                            dim3(256), 0, stream, a);

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "rlk_gemm.hpp"
+#include "rlk_grpo.hpp"
 
 namespace rlk {
 
@@ -235,10 +236,9 @@ struct CombineArgs {
 };
 
 // M = max_s m_s ; S = sum_s s_s 2^(m_s - M) ; z_t = sum_s z_t,s ; lse = ln2 (M + log2 S).
-__global__ void linear_logp_combine_kernel(CombineArgs a)
+// Writes lse and logp of token n and returns the logp.
+__device__ inline float combine_token(const CombineArgs& a, int64_t n)
 {
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
-    if (n >= a.N) return;
     float mm = -INFINITY;
     for (int sp = 0; sp < a.n_split; ++sp) mm = fmaxf(mm, a.part_m[static_cast<int64_t>(sp) * a.N + n]);
     float ss = 0.f, zz = 0.f;
@@ -253,8 +253,65 @@ __global__ void linear_logp_combine_kernel(CombineArgs a)
     const int64_t tl = t - a.vocab_start;
     const bool owned = tl >= 0 && tl < a.V;
     if (!ignored && !owned && a.strict) *a.err_flag = 1;
+    const float lp = ignored ? 0.f : (zz - lse2) * kLn2;
     a.lse[n] = lse2 * kLn2;
-    a.logp[n] = ignored ? 0.f : (zz - lse2) * kLn2;
+    a.logp[n] = lp;
+    return lp;
+}
+
+__global__ void linear_logp_combine_kernel(CombineArgs a)
+{
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= a.N) return;
+    combine_token(a, n);
+}
+
+// Combine with the GRPO loss epilogue folded in: the launch has the block / thread partition of
+// the stand-alone epilogue (block b owns a contiguous token range, thread t walks it with stride
+// 256), merges the split partials of each of its tokens and feeds the fresh log-prob straight into
+// the loss terms, the fixed-order partial sums and d loss / d logp.  The active-token count comes
+// from grpo_count_kernel, which ran before the contraction.  The workgroup that finishes last
+// (integer ticket) adds up the block partials in block order and writes the three scalars, so no
+// further launch is needed.  Same expressions, same partition, same tree as combine +
+// rlk_grpo_loss_from_logp: same bits.
+__global__ __launch_bounds__(kRedThreads) void linear_logp_combine_grpo_kernel(CombineArgs c, GrpoArgs g)
+{
+    const int64_t per = (g.n + g.blocks - 1) / g.blocks;
+    const int64_t lo = per * blockIdx.x;
+    const int64_t hi = lo + per < g.n ? lo + per : g.n;
+    const float denom = grpo_denominator(g.words);
+    Term t{0.f, 0.f, 0.f};
+    for (int64_t i = lo + threadIdx.x; i < hi; i += kRedThreads) {
+        const float lp = combine_token(c, i);
+        const bool on = g.mask == nullptr || g.mask[i] != 0;
+        float r = 0.f, k = 0.f, gr = 0.f, gk = 0.f;
+        if (on) {
+            float pol;
+            token_terms(g, i, lp, r, pol, k);
+            t.pol += pol;
+            if (g.ref_lp != nullptr) t.kl += k;
+            t.act += 1.f;
+            if (g.dcur != nullptr) token_grad(g, i, lp, denom, gr, gk);
+        }
+        if (g.ratio) g.ratio[i] = r;
+        if (g.kl_terms) g.kl_terms[i] = k;
+        if (g.dcur) g.dcur[i] = gr;
+        if (g.dkl) g.dkl[i] = gk;
+    }
+    const Term s = block_sum(t);
+    __shared__ int last_block;
+    if (threadIdx.x == 0) {
+        g.partial[blockIdx.x * 3 + 0] = s.pol;
+        g.partial[blockIdx.x * 3 + 1] = s.kl;
+        g.partial[blockIdx.x * 3 + 2] = s.act;
+        __threadfence();  // the partials are visible before the ticket is taken
+        last_block = atomicAdd(&g.words[0], 1) == g.blocks - 1;
+    }
+    __syncthreads();
+    if (last_block) {  // uniform: every other workgroup has published its partials
+        __threadfence();
+        grpo_finish<true>(g);
+    }
 }
 
 // ------------------------------------------------------------------------------------------- //
@@ -1308,7 +1365,7 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
                 float* logp, float* lse, void* workspace, size_t workspace_bytes, int64_t N,
                 int32_t H, int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
                 int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
-                int32_t* err_flag, hipStream_t stream);
+                int32_t* err_flag, hipStream_t stream, const GrpoArgs* epilogue = nullptr);
 
 }  // namespace
 
@@ -1394,27 +1451,106 @@ int rlk_linear_logp_fwd_static(const void* hidden, const void* weight, const flo
                        strict_targets, err_flag, stream);
 }
 
+int rlk_linear_logp_fwd_grpo_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                                             size_t* bytes)
+{
+    size_t fwd = 0, epi = 0;
+    if (int rc = rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &fwd)) return rc;
+    if (int rc = rlk_grpo_loss_workspace_bytes(N, &epi)) return rc;
+    *bytes = (fwd + 255) / 256 * 256 + epi;
+    return 0;
+}
+
+int rlk_linear_logp_fwd_grpo(const void* hidden, const void* weight, const float* bias,
+                             const int64_t* targets, float* logp, float* lse, void* workspace,
+                             size_t workspace_bytes, int64_t N, int32_t H, int64_t V,
+                             int64_t vocab_start, int32_t dtype, float temperature,
+                             int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
+                             int32_t* err_flag, const float* old_logp, const float* ref_logp,
+                             const float* advantages, int32_t adv_per_token, const uint8_t* mask,
+                             int64_t seq_len, float clip_eps, float beta, float* out3, float* ratio,
+                             float* kl_terms, float* d_cur, float* d_kl, hipStream_t stream)
+{
+    if (int rc = check_common(N, H, V, dtype)) return rc;
+    if (!old_logp || !advantages || !out3 || !logp) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (seq_len <= 0) return rlk_fail(RLK_ERR_ARG, "bad sizes");
+    if (!adv_per_token && N % seq_len != 0)
+        return rlk_fail(RLK_ERR_ARG, "N must be a multiple of seq_len for per-sequence advantages");
+    if (d_kl != nullptr && d_cur == nullptr) return rlk_fail(RLK_ERR_ARG, "d_kl requires d_cur");
+    size_t need = 0, fwd = 0;
+    if (int rc = rlk_linear_logp_fwd_grpo_workspace_bytes(N, H, V, dtype, &need)) return rc;
+    rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &fwd);
+    if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(workspace) & 15) return rlk_fail(RLK_ERR_ARG, "workspace must be 16-byte aligned");
+    GrpoArgs g;
+    g.cur = logp;
+    g.old_lp = old_logp;
+    g.ref_lp = ref_logp;
+    g.adv = advantages;
+    g.mask = mask;
+    g.ratio = ratio;
+    g.kl_terms = kl_terms;
+    g.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + (fwd + 255) / 256 * 256);
+    g.denom = g.partial + kMaxBlocks * 3;
+    g.words = reinterpret_cast<int*>(g.denom + 4);
+    g.out3 = out3;
+    g.dcur = d_cur;
+    g.dkl = d_kl;
+    g.upstream = nullptr;
+    g.n = N;
+    g.seq_len = seq_len;
+    g.adv_per_token = adv_per_token;
+    g.clip_lo = 1.f - clip_eps;
+    g.clip_hi = 1.f + clip_eps;
+    g.beta = beta;
+    g.blocks = grpo_blocks(N);
+    if (!use_mfma(hidden, weight, H, dtype)) {
+        // scalar-FMA forward, then the stand-alone epilogue (same values: it is the same math)
+        if (int rc = fwd_enqueue(hidden, weight, bias, targets, logp, lse, workspace, fwd, N, H, V,
+                                 vocab_start, dtype, temperature, ignore_index, use_ignore,
+                                 strict_targets, err_flag, stream))
+            return rc;
+        return rlk_grpo_loss_from_logp(logp, old_logp, ref_logp, advantages, adv_per_token, mask, N,
+                                       seq_len, clip_eps, beta, out3, ratio, kl_terms, d_cur, d_kl,
+                                       nullptr, g.partial, need - (fwd + 255) / 256 * 256, stream);
+    }
+    return fwd_enqueue(hidden, weight, bias, targets, logp, lse, workspace, fwd, N, H, V, vocab_start,
+                       dtype, temperature, ignore_index, use_ignore, strict_targets, err_flag, stream,
+                       &g);
+}
+
 }  // extern "C"
 
 namespace {
 
+// `epilogue` (optional): GRPO loss arguments whose `cur` is the logp this call produces; the
+// per-token loss pass then runs inside the combine launch.
 int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const int64_t* targets,
                 float* logp, float* lse, void* workspace, size_t workspace_bytes, int64_t N,
                 int32_t H, int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
                 int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
-                int32_t* err_flag, hipStream_t stream)
+                int32_t* err_flag, hipStream_t stream, const GrpoArgs* epilogue)
 {
     if (int rc = check_common(N, H, V, dtype)) return rc;
     if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
     if (!hidden || !weight || !targets || !logp || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
     if (strict_targets && !err_flag)
         return rlk_fail(RLK_ERR_ARG, "strict_targets needs an err_flag to report through");
-    if (!use_mfma(hidden, weight, H, dtype))
+    if (!use_mfma(hidden, weight, H, dtype)) {
+        if (epilogue != nullptr) return rlk_fail(RLK_ERR_UNSUPPORTED, "scalar path has no folded epilogue");
         return generic_fwd(hidden, weight, bias, targets, logp, lse, N, H, V, vocab_start, dtype,
                            temperature, ignore_index, use_ignore, strict_targets, err_flag, stream);
+    }
     size_t need = 0;
     rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &need);
     if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
+    if (epilogue != nullptr) {
+        // the active-token count only needs the mask: it is ready long before the contraction ends
+        const int parts = grpo_count_parts(epilogue->n);
+        hipLaunchKernelGGL(grpo_count_kernel<0>, dim3(parts), dim3(kRedThreads), 0, stream,
+                           epilogue->mask, epilogue->n, parts, epilogue->words);
+        if (int rc = check_launch("grpo_count_kernel launch failed")) return rc;
+    }
 
     FwdArgs a;
     a.hidden = static_cast<const uint16_t*>(hidden);
@@ -1482,8 +1618,13 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
     c.ignore_index = ignore_index;
     c.use_ignore = use_ignore;
     c.strict = strict_targets;
-    hipLaunchKernelGGL(linear_logp_combine_kernel, dim3((a.N + 255) / 256), dim3(256), 0, stream, c);
-    return check_launch("linear_logp_combine_kernel launch failed");
+    if (epilogue == nullptr) {
+        hipLaunchKernelGGL(linear_logp_combine_kernel, dim3((a.N + 255) / 256), dim3(256), 0, stream, c);
+        return check_launch("linear_logp_combine_kernel launch failed");
+    }
+    hipLaunchKernelGGL(linear_logp_combine_grpo_kernel, dim3(epilogue->blocks), dim3(kRedThreads), 0,
+                       stream, c, *epilogue);
+    return check_launch("combine + GRPO epilogue launch failed");
 }
 
 }  // namespace

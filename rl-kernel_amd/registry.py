@@ -35,6 +35,7 @@ class OpBackend(Enum, metaclass=_KernelEnumMeta):
     ROCM_RATIO_KL = "rl_kernel_amd.ops.grpo.RocmRatioKLOp"
     ROCM_GRPO_LOSS = "rl_kernel_amd.ops.grpo.RocmGRPOLossOp"
     ROCM_GRPO_FROM_LOGP = "rl_kernel_amd.ops.grpo.RocmGRPOFromLogpOp"
+    ROCM_GRPO_STEP = "rl_kernel_amd.ops.grpo_step.RocmFusedGRPOStepOp"
 
 
 _LOGP_TYPES = ("logp", "logp_indexed", "logp_online", "logp_online_indexed")
@@ -49,6 +50,7 @@ class KernelRegistry:
             "ratio_kl": [OpBackend.ROCM_RATIO_KL],
             "grpo_loss": [OpBackend.ROCM_GRPO_LOSS],
             "grpo_loss_from_logp": [OpBackend.ROCM_GRPO_FROM_LOGP],
+            "grpo_step_from_hidden": [OpBackend.ROCM_GRPO_STEP],
         }
         for name in _LOGP_TYPES:
             rocm[name] = [OpBackend.ROCM_FUSED_LOGP]

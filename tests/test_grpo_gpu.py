@@ -223,3 +223,70 @@ def test_fused_step_linear_logp_into_grpo_epilogue(dev, ops):
     rel = lambda a, r: ((a.float().cpu() - r).norm() / r.norm()).item()
     assert loss.item() == pytest.approx(loss_ref.item(), abs=1e-4)
     assert rel(hd.grad, dh_ref) < 2e-2 and rel(wd.grad, dw_ref) < 2e-2
+
+
+@pytest.mark.parametrize("b,t,h,v,dtype,per_token_adv,with_ref", [
+    (8, 40, 64, 777, torch.bfloat16, False, True),        # ragged vocab tile, per-sequence advantages
+    (4, 300, 128, 2304, torch.float16, True, True),       # several loss blocks' worth of threads
+    (3, 50, 64, 1000, torch.bfloat16, False, False),      # no reference model: KL term off
+    (64, 512, 256, 4096, torch.bfloat16, False, True),    # 32768 tokens: 8 loss blocks, vocab splits
+])
+def test_epilogue_folded_into_the_forward_equals_the_two_step_route(dev, ops, b, t, h, v, dtype,
+                                                                    per_token_adv, with_ref):
+    """rlk_linear_logp_fwd_grpo = rlk_linear_logp_fwd + rlk_grpo_loss_from_logp, bit for bit:
+    logp, lse, the three scalars, the per-token terms and d loss / d logp; and the op built on it
+    gives the gradients of the two-op composition."""
+    from rl_kernel_amd.ops import linear_logp as LL
+    from rl_kernel_amd.ops.grpo import grpo_from_logp_raw
+    from rl_kernel_amd.ops.grpo_step import RocmFusedGRPOStepOp, fused_linear_logp_grpo_forward
+
+    g = torch.Generator().manual_seed(b * 1000 + t)
+    hidden = torch.randn(b, t, h, generator=g).to(dtype).to(dev)
+    weight = (torch.randn(v, h, generator=g) * 0.1).to(dtype).to(dev)
+    ids = torch.randint(0, v, (b, t), generator=g).to(dev)
+    lens = torch.randint(t // 4, t + 1, (b,), generator=g)
+    mask = (torch.arange(t)[None, :] < lens[:, None]).to(dev)
+    marked = ids.masked_fill(~mask, -100)
+    adv = (torch.randn(b, t, generator=g) if per_token_adv else torch.randn(b, generator=g)).to(dev)
+
+    logp, lse, _ = LL.fused_linear_logp_forward(hidden.view(-1, h), weight, marked.view(-1),
+                                                temperature=0.9, ignore_index=-100)
+    old = (logp + 0.05 * torch.randn(b * t, generator=g).to(dev)).view(b, t)
+    ref = (logp + 0.05 * torch.randn(b * t, generator=g).to(dev)).view(b, t) if with_ref else None
+    out3, ratio, klt, dcur, dkl = grpo_from_logp_raw(logp.view(b, t), old, ref, adv, mask,
+                                                     clip_eps=0.2, beta=0.04, want_grad=True,
+                                                     want_terms=True)
+    f = fused_linear_logp_grpo_forward(hidden.view(-1, h), weight, marked.view(-1), None, old, ref,
+                                       adv, mask, seq_len=t, clip_eps=0.2, beta=0.04,
+                                       temperature=0.9, ignore_index=-100, want_grad=True,
+                                       want_terms=True)
+    f_logp, f_lse, f_err, f_out3, f_ratio, f_klt, f_dcur, f_dkl = f
+    assert int(f_err.item()) == 0
+    assert torch.equal(f_logp, logp) and torch.equal(f_lse, lse)
+    assert torch.equal(f_out3, out3)
+    assert torch.equal(f_ratio, ratio.view(-1)) and torch.equal(f_klt, klt.view(-1))
+    assert torch.equal(f_dcur, dcur.view(-1)) and torch.equal(f_dkl, dkl.view(-1))
+    # against the oracle on the kernel's own log-probs
+    # (without a reference model the KL term is off: the oracle gets ref = cur, whose k3 term is 0)
+    o_loss, o_pol, o_kl, o_dcur = O.grpo_loss_from_logp(
+        logp.view(b, t).cpu(), old.cpu(), (logp.view(b, t) if ref is None else ref).cpu(), adv.cpu(),
+        mask.cpu(), clip_eps=0.2, beta=0.04)
+    assert f_out3[0].item() == pytest.approx(o_loss.item(), abs=2e-5)
+    assert torch.allclose(f_dcur.view(b, t).cpu(), o_dcur, atol=1e-7, rtol=1e-4)
+
+    # the op: same gradients as linear_logp op -> GRPO-from-logp op
+    hd = hidden.clone().requires_grad_(True)
+    wd = weight.clone().requires_grad_(True)
+    loss, pol, kl, cur = RocmFusedGRPOStepOp()(hd, wd, ids, mask, old, ref, adv, clip_eps=0.2,
+                                               beta=0.04, temperature=0.9)
+    assert torch.equal(cur.view(-1), logp) and not cur.requires_grad
+    (loss + 0.5 * kl).backward()
+    hd2 = hidden.clone().requires_grad_(True)
+    wd2 = weight.clone().requires_grad_(True)
+    from rl_kernel_amd.ops.linear_logp import RocmFusedLinearLogpOp
+
+    cur2 = RocmFusedLinearLogpOp()(hd2, wd2, marked, temperature=0.9, ignore_index=-100)
+    loss2, pol2, kl2 = ops.RocmGRPOFromLogpOp()(cur2, old, ref, adv, mask, clip_eps=0.2, beta=0.04)
+    (loss2 + 0.5 * kl2).backward()
+    assert torch.equal(loss, loss2) and torch.equal(pol, pol2) and torch.equal(kl, kl2)
+    assert torch.equal(hd.grad, hd2.grad) and torch.equal(wd.grad, wd2.grad)
