@@ -101,6 +101,27 @@ int rlk_linear_logp_fwd_static(const void* hidden, const void* weight, const flo
                                float temperature, int64_t ignore_index, int32_t use_ignore,
                                int32_t strict_targets, int32_t* err_flag, rlk_stream_t stream);
 
+/* Policy head and frozen reference head over the same hidden states and targets in one launch:
+ * logp / lse of `weight` and ref_logp / ref_lse of `ref_weight` ([V, H], same dtype), each equal
+ * bit for bit to what rlk_linear_logp_fwd returns for that head alone.  A workgroup runs the vocab
+ * tiles of the policy head and then the same tiles of the reference head through one pipeline
+ * against its block of hidden states.  Stands in for the second lm_head pass that yields ref_logps
+ * for the KL term (rl_engine/executors/deepspeed_trainer.py:146-167); the logits-fed counterpart
+ * in the reference is the single program that scans both logit rows
+ * (rl_engine/kernels/ops/triton/loss/ratio_kl.py:46-60).  Only the policy head is strict about
+ * targets; both heads must have a bias or neither.  Workspace: twice the single-head size
+ * (rlk_linear_logp_fwd_pair_workspace_bytes). */
+int rlk_linear_logp_fwd_pair_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                                             size_t* bytes);
+
+int rlk_linear_logp_fwd_pair(const void* hidden, const void* weight, const void* ref_weight,
+                             const float* bias, const float* ref_bias, const int64_t* targets,
+                             float* logp, float* lse, float* ref_logp, float* ref_lse,
+                             void* workspace, size_t workspace_bytes, int64_t N, int32_t H,
+                             int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                             int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
+                             int32_t* err_flag, rlk_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------ *
  * Fused linear -> log-prob, backward.
  *
@@ -153,6 +174,15 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
 int rlk_logp_from_logits(const void* logits, int32_t logits_dtype, const int64_t* ids, void* out,
                          int32_t out_dtype, float* lse_out, const int64_t* row_indices,
                          int64_t n_launch, int64_t n_rows, int64_t vocab, rlk_stream_t stream);
+
+/* The same scan over two logits tensors of one shape and dtype (policy and reference) with shared
+ * ids and row list in ONE launch, as the reference's ratio/KL program reads both rows
+ * (rl_engine/kernels/ops/triton/loss/ratio_kl.py:46-60).  Each output equals the single call bit
+ * for bit. */
+int rlk_logp_from_logits_pair(const void* logits, const void* ref_logits, int32_t logits_dtype,
+                              const int64_t* ids, void* out, void* ref_out, int32_t out_dtype,
+                              float* lse_out, float* ref_lse_out, const int64_t* row_indices,
+                              int64_t n_launch, int64_t n_rows, int64_t vocab, rlk_stream_t stream);
 
 /* Backward of the above w.r.t. the logits:
  *   grad_logits[n][v] = coeff[n] * (onehot(ids[n])[v] - exp(logits[n][v] - lse[n]))

@@ -29,6 +29,13 @@ struct FwdArgs {
     float* part_m;            // [n_split][N] running max (log2 domain)
     float* part_s;            // [n_split][N] running sum of 2^(z - max)
     float* part_z;            // [n_split][N] captured target logit (log2 domain), 0 if not owned
+    // optional second head over the same hidden states and targets (a frozen reference model):
+    // its tiles follow the first head's in the same pipeline, its partials go to part2_*
+    const uint16_t* weight2;  // [V][H] or null
+    const float* bias2;       // [V] or null
+    float* part2_m;
+    float* part2_s;
+    float* part2_z;
     int N;
     int H;
     int V;
@@ -46,15 +53,15 @@ struct FwdArgs {
 // The target logit is picked up in the same pass that feeds the sum, so the captured value is
 // the very fp32 number that entered the softmax.
 template <bool GENERAL>
-__device__ inline void fwd_epilogue(const f32x16_t (&acc)[kTM][kTN], const FwdArgs& a, int vw,
-                                    int lane, const int (&tgt)[kTN], float (&m)[kTN],
-                                    float (&s)[kTN], float (&zt)[kTN])
+__device__ inline void fwd_epilogue(const f32x16_t (&acc)[kTM][kTN], const FwdArgs& a,
+                                    const float* bias, int vw, int lane, const int (&tgt)[kTN],
+                                    float (&m)[kTN], float (&s)[kTN], float (&zt)[kTN])
 {
     auto logit = [&](int i, int j, int r) -> float {
         float z = acc[i][j][r];
         if (GENERAL) {
             const int v = vw + i * 32 + acc_row(r, lane);
-            if (a.bias != nullptr) z += a.bias[v < a.V ? v : a.V - 1];
+            if (bias != nullptr) z += bias[v < a.V ? v : a.V - 1];
             if (v >= a.V) z = -INFINITY;
         }
         return z;
@@ -131,90 +138,124 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
     int tgt[TN];  // target id relative to the shard, -1 when not in [0, V)
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        m[j] = -INFINITY;
-        s[j] = 0.f;
-        zt[j] = 0.f;
         const int t = wn * (TN * 32) + j * 32 + (lane & 31);
         int64_t g = a.targets[tok0 + (t < tok_valid ? t : tok_valid - 1)] - a.vocab_start;
         tgt[j] = (g >= 0 && g < a.V) ? static_cast<int>(g) : -1;
     }
+    auto reset_state = [&]() {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            m[j] = -INFINITY;
+            s[j] = 0.f;
+            zt[j] = 0.f;
+        }
+    };
 
+    // Merge of one head's state: the two half-wave row groups (same token, different vocab rows),
+    // then the wavefronts along M through LDS, in a fixed order; written to that head's partial
+    // arrays.  The LDS patch lies behind the pipeline stages, so the merge of the first head can run
+    // while the second head's first K steps are already on their way.
+    float* red = reinterpret_cast<float*>(smem + TileGemmDtl<T, false, false, BK>::kSmemBytes);  // [kWM][256 tokens][3]
+    static_assert(TileGemmDtl<T, false, false, BK>::kSmemBytes + kWM * 256 * 3 * 4 <= Gemm::kSmemBytes,
+                  "merge patch must fit the kernel's LDS");
+    auto flush_state = [&](float* pm, float* ps, float* pz) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const float m2 = __shfl_xor(m[j], 32);
+            const float s2 = __shfl_xor(s[j], 32);
+            const float z2 = __shfl_xor(zt[j], 32);
+            const float mm = fmaxf(m[j], m2);
+            const float mref = mm == -INFINITY ? 0.f : mm;
+            const float lo_m = lane < 32 ? m[j] : m2, hi_m = lane < 32 ? m2 : m[j];
+            const float lo_s = lane < 32 ? s[j] : s2, hi_s = lane < 32 ? s2 : s[j];
+            const float ss = lo_s * __builtin_amdgcn_exp2f(lo_m - mref) +
+                             hi_s * __builtin_amdgcn_exp2f(hi_m - mref);
+            if (lane < 32) {
+                float* dst = red + ((wm * 256) + wn * (TN * 32) + j * 32 + lane) * 3;
+                dst[0] = mm;
+                dst[1] = ss;
+                dst[2] = zt[j] + z2;
+            }
+        }
+        __syncthreads();
+        const int t = threadIdx.x;
+        if (t < tok_valid) {
+            float mm = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < kWM; ++w) mm = fmaxf(mm, red[(w * 256 + t) * 3]);
+            const float mref = mm == -INFINITY ? 0.f : mm;
+            float ss = 0.f, zz = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWM; ++w) {
+                const float* pw = red + (w * 256 + t) * 3;
+                ss += pw[1] * __builtin_amdgcn_exp2f(pw[0] - mref);
+                zz += pw[2];
+            }
+            const int64_t o = static_cast<int64_t>(a.split_lo + sp) * a.N + tok0 + t;
+            pm[o] = mm;
+            ps[o] = ss;
+            pz[o] = zz;
+        }
+        __syncthreads();  // the patch may be written again
+    };
+
+    const int n_heads = a.weight2 != nullptr ? 2 : 1;
     Operand B{a.hidden + static_cast<int64_t>(tok0) * a.H, a.H, tok_valid};
-    auto tile_origin = [&](int vt) { return a.weight + static_cast<int64_t>(vt) * 256 * a.H; };
+    auto tile_origin = [&](int head, int vt) {
+        return (head == 0 ? a.weight : a.weight2) + static_cast<int64_t>(vt) * 256 * a.H;
+    };
     if (!GENERAL && RLK_DTL != 0 && RLK_STREAM != 0 && a.H % BK == 0 && a.H >= 2 * BK && t0 < t1) {
-        // every tile is full: one pipeline runs through all tiles of the range, the K loop of a
-        // tile already fetching the head of the next one while the softmax update runs (the
-        // pipeline looks two K steps ahead, which stays within the next tile from two steps up)
+        // every tile is full: one pipeline runs through all tiles of the range (and then through
+        // the same range of the second head), the K loop of a tile already fetching the head of the
+        // next one while the softmax update runs (the pipeline looks two K steps ahead, which stays
+        // within the next tile from two steps up)
         using Dtl = TileGemmDtl<T, false, false, BK>;
         typename Dtl::Stream st;
-        Dtl::begin(st, Operand{tile_origin(t0), a.H, 256}, B, a.H, smem);
-        for (int vt = t0; vt < t1; ++vt) {
-            f32x16_t acc[TM][TN];
+        Dtl::begin(st, Operand{tile_origin(0, t0), a.H, 256}, B, a.H, smem);
+        for (int head = 0; head < n_heads; ++head) {
+            reset_state();
+            for (int vt = t0; vt < t1; ++vt) {
+                f32x16_t acc[TM][TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                    for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-            Dtl::tile(st, tile_origin(vt + 1 < t1 ? vt + 1 : vt), B.base, acc, smem);
-            fwd_epilogue<GENERAL>(acc, a, vt * 256 + wm * (TM * 32), lane, tgt, m, s, zt);
+                        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+                const void* next = vt + 1 < t1 ? tile_origin(head, vt + 1)
+                                               : (head + 1 < n_heads ? tile_origin(head + 1, t0)
+                                                                     : tile_origin(head, vt));
+                Dtl::tile(st, next, B.base, acc, smem);
+                fwd_epilogue<GENERAL>(acc, a, nullptr, vt * 256 + wm * (TM * 32), lane, tgt, m, s, zt);
+            }
+            if (head == 0)
+                flush_state(a.part_m, a.part_s, a.part_z);
+            else
+                flush_state(a.part2_m, a.part2_s, a.part2_z);
         }
         Dtl::end(st);
     } else {
-        for (int vt = t0; vt < t1; ++vt) {
-            const int v0 = vt * 256;
-            Operand A{tile_origin(vt), a.H, min(256, a.V - v0)};
-            f32x16_t acc[TM][TN];
+        for (int head = 0; head < n_heads; ++head) {
+            reset_state();
+            const float* bias = head == 0 ? a.bias : a.bias2;
+            for (int vt = t0; vt < t1; ++vt) {
+                const int v0 = vt * 256;
+                Operand A{tile_origin(head, vt), a.H, min(256, a.V - v0)};
+                f32x16_t acc[TM][TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                    for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-            Gemm::run(A, B, a.H, acc, smem);
-            fwd_epilogue<GENERAL>(acc, a, v0 + wm * (TM * 32), lane, tgt, m, s, zt);
+                        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+                Gemm::run(A, B, a.H, acc, smem);
+                fwd_epilogue<GENERAL>(acc, a, bias, v0 + wm * (TM * 32), lane, tgt, m, s, zt);
+            }
+            if (head == 0)
+                flush_state(a.part_m, a.part_s, a.part_z);
+            else
+                flush_state(a.part2_m, a.part2_s, a.part2_z);
         }
-    }
-
-    // Merge the two half-wave row groups (same token, different vocab rows), then the two
-    // wavefronts along M through LDS, in a fixed order.
-    float* red = reinterpret_cast<float*>(smem);  // [kWM][256 tokens][3]
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const float m2 = __shfl_xor(m[j], 32);
-        const float s2 = __shfl_xor(s[j], 32);
-        const float z2 = __shfl_xor(zt[j], 32);
-        const float mm = fmaxf(m[j], m2);
-        const float mref = mm == -INFINITY ? 0.f : mm;
-        const float lo_m = lane < 32 ? m[j] : m2, hi_m = lane < 32 ? m2 : m[j];
-        const float lo_s = lane < 32 ? s[j] : s2, hi_s = lane < 32 ? s2 : s[j];
-        const float ss = lo_s * __builtin_amdgcn_exp2f(lo_m - mref) +
-                         hi_s * __builtin_amdgcn_exp2f(hi_m - mref);
-        if (lane < 32) {
-            float* dst = red + ((wm * 256) + wn * (TN * 32) + j * 32 + lane) * 3;
-            dst[0] = mm;
-            dst[1] = ss;
-            dst[2] = zt[j] + z2;
-        }
-    }
-    __syncthreads();
-    const int t = threadIdx.x;
-    if (t < tok_valid) {
-        float mm = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < kWM; ++w) mm = fmaxf(mm, red[(w * 256 + t) * 3]);
-        const float mref = mm == -INFINITY ? 0.f : mm;
-        float ss = 0.f, zz = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWM; ++w) {
-            const float* pw = red + (w * 256 + t) * 3;
-            ss += pw[1] * __builtin_amdgcn_exp2f(pw[0] - mref);
-            zz += pw[2];
-        }
-        const int64_t o = static_cast<int64_t>(a.split_lo + sp) * a.N + tok0 + t;
-        a.part_m[o] = mm;
-        a.part_s[o] = ss;
-        a.part_z[o] = zz;
     }
 }
 
@@ -1361,11 +1402,20 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
     return 0;
 }
 
+// A second head over the same hidden states and targets (a frozen reference model).
+struct SecondHead {
+    const void* weight;
+    const float* bias;
+    float* logp;
+    float* lse;
+};
+
 int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const int64_t* targets,
                 float* logp, float* lse, void* workspace, size_t workspace_bytes, int64_t N,
                 int32_t H, int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
                 int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
-                int32_t* err_flag, hipStream_t stream, const GrpoArgs* epilogue = nullptr);
+                int32_t* err_flag, hipStream_t stream, const GrpoArgs* epilogue = nullptr,
+                const SecondHead* second = nullptr);
 
 }  // namespace
 
@@ -1451,6 +1501,31 @@ int rlk_linear_logp_fwd_static(const void* hidden, const void* weight, const flo
                        strict_targets, err_flag, stream);
 }
 
+int rlk_linear_logp_fwd_pair_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                                             size_t* bytes)
+{
+    if (int rc = rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, bytes)) return rc;
+    *bytes *= 2;
+    return 0;
+}
+
+int rlk_linear_logp_fwd_pair(const void* hidden, const void* weight, const void* ref_weight,
+                             const float* bias, const float* ref_bias, const int64_t* targets,
+                             float* logp, float* lse, float* ref_logp, float* ref_lse,
+                             void* workspace, size_t workspace_bytes, int64_t N, int32_t H,
+                             int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                             int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
+                             int32_t* err_flag, hipStream_t stream)
+{
+    if (!ref_weight || !ref_logp || !ref_lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if ((bias == nullptr) != (ref_bias == nullptr))
+        return rlk_fail(RLK_ERR_UNSUPPORTED, "both heads must have a bias or neither");
+    const SecondHead second{ref_weight, ref_bias, ref_logp, ref_lse};
+    return fwd_enqueue(hidden, weight, bias, targets, logp, lse, workspace, workspace_bytes, N, H, V,
+                       vocab_start, dtype, temperature, ignore_index, use_ignore, strict_targets,
+                       err_flag, stream, nullptr, &second);
+}
+
 int rlk_linear_logp_fwd_grpo_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                              size_t* bytes)
 {
@@ -1529,20 +1604,29 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
                 float* logp, float* lse, void* workspace, size_t workspace_bytes, int64_t N,
                 int32_t H, int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
                 int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
-                int32_t* err_flag, hipStream_t stream, const GrpoArgs* epilogue)
+                int32_t* err_flag, hipStream_t stream, const GrpoArgs* epilogue,
+                const SecondHead* second)
 {
     if (int rc = check_common(N, H, V, dtype)) return rc;
     if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
     if (!hidden || !weight || !targets || !logp || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
     if (strict_targets && !err_flag)
         return rlk_fail(RLK_ERR_ARG, "strict_targets needs an err_flag to report through");
-    if (!use_mfma(hidden, weight, H, dtype)) {
+    const bool mfma = use_mfma(hidden, weight, H, dtype) &&
+                      (second == nullptr || use_mfma(hidden, second->weight, H, dtype));
+    if (!mfma) {
         if (epilogue != nullptr) return rlk_fail(RLK_ERR_UNSUPPORTED, "scalar path has no folded epilogue");
-        return generic_fwd(hidden, weight, bias, targets, logp, lse, N, H, V, vocab_start, dtype,
-                           temperature, ignore_index, use_ignore, strict_targets, err_flag, stream);
+        if (int rc = generic_fwd(hidden, weight, bias, targets, logp, lse, N, H, V, vocab_start, dtype,
+                                 temperature, ignore_index, use_ignore, strict_targets, err_flag, stream))
+            return rc;
+        if (second == nullptr) return 0;
+        return generic_fwd(hidden, second->weight, second->bias, targets, second->logp, second->lse, N,
+                           H, V, vocab_start, dtype, temperature, ignore_index, use_ignore, 0,
+                           err_flag, stream);
     }
     size_t need = 0;
     rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &need);
+    if (second != nullptr) need *= 2;
     if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
     if (epilogue != nullptr) {
         // the active-token count only needs the mask: it is ready long before the contraction ends
@@ -1556,16 +1640,22 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
     a.hidden = static_cast<const uint16_t*>(hidden);
     a.weight = static_cast<const uint16_t*>(weight);
     a.bias = bias;
+    a.weight2 = second ? static_cast<const uint16_t*>(second->weight) : nullptr;
+    a.bias2 = second ? second->bias : nullptr;
     a.targets = targets;
     a.N = static_cast<int>(N);
     a.H = H;
     a.V = static_cast<int>(V);
     a.vocab_start = vocab_start;
-    const FwdPlan plan = fwd_plan(N, V, bias != nullptr);
+    // with two heads a bias on either sends both through the general launch
+    const FwdPlan plan = fwd_plan(N, V, bias != nullptr || (second != nullptr && second->bias != nullptr));
     a.row_blocks = plan.row_blocks;
     a.part_m = static_cast<float*>(workspace);
     a.part_s = a.part_m + static_cast<size_t>(plan.total_splits) * N;
     a.part_z = a.part_s + static_cast<size_t>(plan.total_splits) * N;
+    a.part2_m = a.part_z + static_cast<size_t>(plan.total_splits) * N;
+    a.part2_s = a.part2_m + static_cast<size_t>(plan.total_splits) * N;
+    a.part2_z = a.part2_s + static_cast<size_t>(plan.total_splits) * N;
     a.scale2 = kLog2e / temperature;
 
     using G = TileGemm<Bf16, false, false, kBK>;  // same LDS footprint for f16
@@ -1618,6 +1708,16 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
     c.ignore_index = ignore_index;
     c.use_ignore = use_ignore;
     c.strict = strict_targets;
+    if (second != nullptr) {  // the reference head: same merge, never strict
+        CombineArgs c2 = c;
+        c2.part_m = a.part2_m;
+        c2.part_s = a.part2_s;
+        c2.part_z = a.part2_z;
+        c2.logp = second->logp;
+        c2.lse = second->lse;
+        c2.strict = 0;
+        hipLaunchKernelGGL(linear_logp_combine_kernel, dim3((a.N + 255) / 256), dim3(256), 0, stream, c2);
+    }
     if (epilogue == nullptr) {
         hipLaunchKernelGGL(linear_logp_combine_kernel, dim3((a.N + 255) / 256), dim3(256), 0, stream, c);
         return check_launch("linear_logp_combine_kernel launch failed");

@@ -65,12 +65,24 @@ __device__ inline void store_out(void* out, int dtype, int64_t i, float v)
 
 constexpr int kScanThreads = 256;
 
+// Second logits tensor of a pair launch (grid.y == 2): same ids and rows, own outputs.
+struct ScanSecond {
+    const void* logits;
+    void* out;
+    float* lse_out;
+};
+
 template <int DT>
 __global__ __launch_bounds__(kScanThreads) void logp_scan_kernel(
     const void* __restrict__ logits_v, const int64_t* __restrict__ ids, void* __restrict__ out,
     int out_dtype, float* __restrict__ lse_out, const int64_t* __restrict__ row_indices,
-    int64_t n_rows, int64_t vocab)
+    int64_t n_rows, int64_t vocab, ScanSecond second)
 {
+    if (blockIdx.y == 1) {  // uniform
+        logits_v = second.logits;
+        out = second.out;
+        lse_out = second.lse_out;
+    }
     using E = typename Elem<DT>::type;
     constexpr int kPer = 16 / sizeof(E);  // elements per 16-byte load
     const int64_t row = row_indices ? row_indices[blockIdx.x] : static_cast<int64_t>(blockIdx.x);
@@ -237,34 +249,61 @@ extern "C" int rlk_logp_from_logits_bwd(const void* logits, int32_t logits_dtype
 }
 
 
-extern "C" int rlk_logp_from_logits(const void* logits, int32_t logits_dtype, const int64_t* ids,
-                                    void* out, int32_t out_dtype, float* lse_out,
-                                    const int64_t* row_indices, int64_t n_launch, int64_t n_rows,
-                                    int64_t vocab, hipStream_t stream)
+namespace {
+
+int scan_enqueue(const void* logits, int32_t logits_dtype, const int64_t* ids, void* out,
+                 int32_t out_dtype, float* lse_out, const int64_t* row_indices, int64_t n_launch,
+                 int64_t n_rows, int64_t vocab, const rlk::ScanSecond* second, hipStream_t stream)
 {
+    using namespace rlk;
     if (!logits || !ids || !out) return rlk_fail(RLK_ERR_ARG, "null pointer");
     if (n_rows < 0 || vocab <= 0 || n_launch < 0) return rlk_fail(RLK_ERR_ARG, "bad sizes");
     if (n_launch > 0x7fffffffLL) return rlk_fail(RLK_ERR_ARG, "too many rows for one launch");
     if (out_dtype < RLK_DTYPE_BF16 || out_dtype > RLK_DTYPE_F64)
         return rlk_fail(RLK_ERR_UNSUPPORTED, "output dtype must be bf16, f16, f32 or f64");
     if (n_launch == 0 || n_rows == 0) return 0;
-    const dim3 grid(static_cast<unsigned>(n_launch)), block(kScanThreads);
+    const dim3 grid(static_cast<unsigned>(n_launch), second ? 2u : 1u), block(kScanThreads);
+    const ScanSecond s2 = second ? *second : ScanSecond{nullptr, nullptr, nullptr};
     switch (logits_dtype) {
         case RLK_DTYPE_BF16:
             hipLaunchKernelGGL(logp_scan_kernel<RLK_DTYPE_BF16>, grid, block, 0, stream, logits, ids,
-                               out, out_dtype, lse_out, row_indices, n_rows, vocab);
+                               out, out_dtype, lse_out, row_indices, n_rows, vocab, s2);
             break;
         case RLK_DTYPE_F16:
             hipLaunchKernelGGL(logp_scan_kernel<RLK_DTYPE_F16>, grid, block, 0, stream, logits, ids,
-                               out, out_dtype, lse_out, row_indices, n_rows, vocab);
+                               out, out_dtype, lse_out, row_indices, n_rows, vocab, s2);
             break;
         case RLK_DTYPE_F32:
             hipLaunchKernelGGL(logp_scan_kernel<RLK_DTYPE_F32>, grid, block, 0, stream, logits, ids,
-                               out, out_dtype, lse_out, row_indices, n_rows, vocab);
+                               out, out_dtype, lse_out, row_indices, n_rows, vocab, s2);
             break;
         default:
             return rlk_fail(RLK_ERR_UNSUPPORTED, "logits dtype must be bf16, f16 or f32");
     }
     if (hipGetLastError() != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, "logp scan launch failed");
     return 0;
+}
+
+}  // namespace
+
+extern "C" int rlk_logp_from_logits(const void* logits, int32_t logits_dtype, const int64_t* ids,
+                                    void* out, int32_t out_dtype, float* lse_out,
+                                    const int64_t* row_indices, int64_t n_launch, int64_t n_rows,
+                                    int64_t vocab, hipStream_t stream)
+{
+    return scan_enqueue(logits, logits_dtype, ids, out, out_dtype, lse_out, row_indices, n_launch,
+                        n_rows, vocab, nullptr, stream);
+}
+
+extern "C" int rlk_logp_from_logits_pair(const void* logits, const void* ref_logits,
+                                         int32_t logits_dtype, const int64_t* ids, void* out,
+                                         void* ref_out, int32_t out_dtype, float* lse_out,
+                                         float* ref_lse_out, const int64_t* row_indices,
+                                         int64_t n_launch, int64_t n_rows, int64_t vocab,
+                                         hipStream_t stream)
+{
+    if (!ref_logits || !ref_out) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    const rlk::ScanSecond second{ref_logits, ref_out, ref_lse_out};
+    return scan_enqueue(logits, logits_dtype, ids, out, out_dtype, lse_out, row_indices, n_launch,
+                        n_rows, vocab, &second, stream);
 }

@@ -17,7 +17,7 @@ import torch
 
 from .. import _native
 from ..platform import logger
-from .logp import differentiable_logp_fp32
+from .logp import differentiable_logp_pair_fp32
 
 
 def _stream(device):
@@ -178,9 +178,9 @@ class RocmRatioKLOp:
             raise ValueError(f"action_ids at active (unmasked) positions must be in "
                              f"[0, {vocab}); found out-of-range ids.")
         safe_ids = action_ids.masked_fill(~mask, 0)
-        logp_policy = differentiable_logp_fp32(policy_logits, safe_ids)
-        with torch.no_grad():
-            logp_ref = differentiable_logp_fp32(ref_logits.detach(), safe_ids)
+        # both logit tensors in one scan launch (the reference's program reads both rows too:
+        # rl_engine/kernels/ops/triton/loss/ratio_kl.py:46-60)
+        logp_policy, logp_ref = differentiable_logp_pair_fp32(policy_logits, ref_logits, safe_ids)
         delta = (logp_policy - old_logps.float()).masked_fill(~mask, 0.0)
         diff = (logp_ref - logp_policy).masked_fill(~mask, 0.0)
         return torch.exp(delta), torch.exp(diff) - diff - 1.0
@@ -222,9 +222,7 @@ class RocmGRPOLossOp:
             raise ValueError(f"action_ids at active (unmasked) positions must be in "
                              f"[0, {vocab}); found out-of-range ids.")
         safe_ids = action_ids.masked_fill(~mask, 0)
-        cur = differentiable_logp_fp32(policy_logits, safe_ids)
-        with torch.no_grad():
-            ref = differentiable_logp_fp32(ref_logits.detach(), safe_ids)
+        cur, ref = differentiable_logp_pair_fp32(policy_logits, ref_logits, safe_ids)
         return self._from_logp(cur, old_logps, ref, sample_advantages.reshape(-1), mask,
                                clip_eps=clip_eps, beta=beta)
 

@@ -120,6 +120,50 @@ def fused_linear_logp_forward(
     return logp, lse, err
 
 
+def fused_linear_logp_forward_pair(
+    hidden_2d: torch.Tensor,
+    weight: torch.Tensor,
+    ref_weight: torch.Tensor,
+    target_1d: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    ref_bias: Optional[torch.Tensor] = None,
+    *,
+    temperature: float = 1.0,
+    ignore_index: Optional[int] = None,
+    vocab_start: int = 0,
+    strict_targets: bool = True,
+):
+    """Policy head and frozen reference head in one launch: ``(logp, lse, ref_logp, ref_lse,
+    err_flag)``, each pair equal bit for bit to ``fused_linear_logp_forward`` on that head."""
+    lib = _native.load()
+    n, h = hidden_2d.shape
+    v = weight.size(0)
+    if ref_weight.shape != weight.shape or ref_weight.dtype != weight.dtype:
+        raise ValueError(f"reference weight {tuple(ref_weight.shape)} {ref_weight.dtype} must match "
+                         f"the policy weight {tuple(weight.shape)} {weight.dtype}")
+    dev = hidden_2d.device
+    outs = [torch.empty(n, device=dev, dtype=torch.float32) for _ in range(4)]
+    err = torch.zeros(1, device=dev, dtype=torch.int32)
+    if n == 0:
+        return (*outs, err)
+    _warn_if_scalar_path(hidden_2d, weight)
+    need = _native.ctypes.c_size_t(0)
+    dt = _DTYPES[hidden_2d.dtype]
+    _native.check(lib.rlk_linear_logp_fwd_pair_workspace_bytes(n, h, v, dt, _native.ctypes.byref(need)),
+                  "linear_logp pair workspace query")
+    ws = torch.empty(max(need.value, 16), device=dev, dtype=torch.uint8)
+    f32 = lambda b: None if b is None else b.detach().to(torch.float32).contiguous()
+    bias_f, ref_bias_f = f32(bias), f32(ref_bias)
+    rc = lib.rlk_linear_logp_fwd_pair(
+        _ptr(hidden_2d), _ptr(weight), _ptr(ref_weight), _ptr(bias_f), _ptr(ref_bias_f),
+        _ptr(target_1d), _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(outs[3]), _ptr(ws),
+        ws.numel(), n, h, v, int(vocab_start), dt, float(temperature),
+        0 if ignore_index is None else int(ignore_index), int(ignore_index is not None),
+        int(strict_targets), _ptr(err), _stream(dev))
+    _native.check(rc, "rlk_linear_logp_fwd_pair")
+    return (*outs, err)
+
+
 def fused_linear_logp_backward(
     grad_logp: torch.Tensor,
     hidden_2d: torch.Tensor,
@@ -216,6 +260,39 @@ class _FusedLinearLogpFunction(torch.autograd.Function):
         return grad_hidden, grad_weight, grad_bias, None, None, None, None
 
 
+class _FusedLinearLogpPairFunction(torch.autograd.Function):
+    """Policy log-probs (differentiable) and reference log-probs (no gradient) from one launch."""
+
+    @staticmethod
+    def forward(ctx, hidden, weight, bias, ref_weight, ref_bias, target_ids, temperature,
+                ignore_index, check_targets):
+        hidden_2d = _aligned_contiguous(hidden.reshape(-1, hidden.size(-1)))
+        w = _aligned_contiguous(weight)
+        w_ref = _aligned_contiguous(ref_weight.detach())
+        target_1d = target_ids.reshape(-1).to(device=hidden_2d.device, dtype=torch.long).contiguous()
+        logp, lse, ref_logp, _, err = fused_linear_logp_forward_pair(
+            hidden_2d, w, w_ref, target_1d, bias, ref_bias, temperature=temperature,
+            ignore_index=ignore_index)
+        if check_targets and hidden_2d.size(0) > 0 and bool(err.item()):
+            raise _out_of_range_error(target_1d, w.size(0), ignore_index)
+        ctx.empty = hidden_2d.size(0) == 0
+        ctx.save_for_backward(hidden_2d, w, bias if bias is not None else hidden_2d, target_1d, lse)
+        ctx.has_bias = bias is not None
+        ctx.lead_shape = hidden.shape[:-1]
+        ctx.temperature = temperature
+        ctx.ignore_index = ignore_index
+        ctx.weight_dtype = weight.dtype
+        ctx.bias_dtype = bias.dtype if bias is not None else None
+        ref_out = ref_logp.reshape(hidden.shape[:-1])
+        ctx.mark_non_differentiable(ref_out)
+        return logp.reshape(hidden.shape[:-1]), ref_out
+
+    @staticmethod
+    def backward(ctx, grad_logp, _grad_ref):
+        grads = _FusedLinearLogpFunction.backward(ctx, grad_logp)
+        return grads[0], grads[1], grads[2], None, None, None, None, None, None
+
+
 class RocmFusedLinearLogpOp:
     """gfx950 MFMA fused linear log-prob: ``log_softmax((hidden W^T + b)/T)[target]`` without the
     ``[N, V]`` logits.  Constructor raises ``RuntimeError`` when the HIP library or a ROCm GPU is
@@ -283,3 +360,34 @@ class RocmFusedLinearLogpOp:
                 "(bf16, f16 or f32) on the same GPU")
         return _FusedLinearLogpFunction.apply(hidden, lm_head_weight, bias, target_ids,
                                               float(temperature), ignore_index, check_targets)
+
+    def with_reference(self, hidden, lm_head_weight, ref_lm_head_weight, target_ids, bias=None,
+                       ref_bias=None, *, temperature: float = 1.0,
+                       ignore_index: Optional[int] = None, check_targets: bool = True):
+        """``(logp, ref_logp)``: the policy head and a frozen reference head over the same hidden
+        states and targets in one launch (the reference log-probs the KL term needs, which the
+        trainer otherwise gets from a second lm_head pass).  ``logp`` is differentiable w.r.t.
+        hidden, weight and bias; ``ref_logp`` carries no gradient.  Each equals what ``apply``
+        returns for that head, bit for bit."""
+        if temperature <= 0.0:
+            raise ValueError("temperature must be greater than zero")
+        if lm_head_weight.size(-1) != hidden.size(-1):
+            raise ValueError(f"hidden dim {hidden.size(-1)} must match lm_head_weight dim "
+                             f"{lm_head_weight.size(-1)}")
+        if ref_lm_head_weight.shape != lm_head_weight.shape:
+            raise ValueError(f"reference weight shape {tuple(ref_lm_head_weight.shape)} must match "
+                             f"lm_head_weight shape {tuple(lm_head_weight.shape)}")
+        if hidden.shape[:-1] != target_ids.shape:
+            raise ValueError(f"hidden leading shape {tuple(hidden.shape[:-1])} must match "
+                             f"target_ids shape {tuple(target_ids.shape)}")
+        if (bias is None) != (ref_bias is None):
+            raise ValueError("both heads must have a bias or neither")
+        if not hip_path_supported(hidden, lm_head_weight) or \
+                ref_lm_head_weight.dtype != lm_head_weight.dtype or \
+                ref_lm_head_weight.device != lm_head_weight.device:
+            raise NotImplementedError(
+                "with_reference needs hidden and both weights of one dtype (bf16, f16 or f32) on "
+                "the same GPU")
+        return _FusedLinearLogpPairFunction.apply(hidden, lm_head_weight, bias, ref_lm_head_weight,
+                                                  ref_bias, target_ids, float(temperature),
+                                                  ignore_index, check_targets)

@@ -181,6 +181,52 @@ class _LogpFromLogitsFunction(torch.autograd.Function):
         return grad.view(ctx.logits_shape), None
 
 
+class _LogpPairFromLogitsFunction(torch.autograd.Function):
+    """fp32 selected log-probs of a policy and a reference logits tensor from ONE scan launch;
+    differentiable w.r.t. the policy logits only."""
+
+    @staticmethod
+    def forward(ctx, logits, ref_logits, ids):
+        shape = logits.shape[:-1]
+        logits_2d = logits.reshape(-1, logits.size(-1)).contiguous()
+        ref_2d = ref_logits.reshape(-1, ref_logits.size(-1)).contiguous()
+        ids_1d = ids.reshape(-1).to(device=logits.device, dtype=torch.long).contiguous()
+        n, v = logits_2d.shape
+        out = torch.empty(n, device=logits.device, dtype=torch.float32)
+        ref_out = torch.empty(n, device=logits.device, dtype=torch.float32)
+        lse = torch.empty(n, device=logits.device, dtype=torch.float32)
+        if n > 0:
+            rc = _native.load().rlk_logp_from_logits_pair(
+                logits_2d.data_ptr(), ref_2d.data_ptr(), _IN[logits_2d.dtype], ids_1d.data_ptr(),
+                out.data_ptr(), ref_out.data_ptr(), _OUT[torch.float32], lse.data_ptr(), None, None,
+                n, n, v, _stream(logits_2d.device))
+            _native.check(rc, "rlk_logp_from_logits_pair")
+        ctx.save_for_backward(logits_2d, ids_1d, lse)
+        ctx.logits_shape = logits.shape
+        ref_view = ref_out.view(shape)
+        ctx.mark_non_differentiable(ref_view)
+        return out.view(shape), ref_view
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_ref):
+        grad, _ = _LogpFromLogitsFunction.backward(ctx, grad_out)
+        return grad, None, None
+
+
+def differentiable_logp_pair_fp32(logits: torch.Tensor, ref_logits: torch.Tensor,
+                                  ids: torch.Tensor):
+    """``(logp_policy, logp_ref)``; one launch when both tensors share shape, dtype and device,
+    two scans otherwise."""
+    if logits.dtype not in _IN or ref_logits.dtype not in _IN:
+        raise RuntimeError("logits dtype must be float32, float16 or bfloat16")
+    if (logits.shape == ref_logits.shape and logits.dtype == ref_logits.dtype
+            and logits.device == ref_logits.device):
+        return _LogpPairFromLogitsFunction.apply(logits, ref_logits.detach(), ids)
+    with torch.no_grad():
+        ref = _LogpFromLogitsFunction.apply(ref_logits.detach(), ids)
+    return _LogpFromLogitsFunction.apply(logits, ids), ref
+
+
 def differentiable_logp_fp32(logits: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     if logits.dtype not in _IN:
         raise RuntimeError("logits dtype must be float32, float16 or bfloat16")
