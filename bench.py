@@ -466,6 +466,37 @@ def bench_registry_op(torch, hidden, weight, targets, grad, temp, ign, steps):
                     "reference's backward keeps an fp32 grad_w) and the saved lse"}
 
 
+def bench_variants(torch, cfg):
+    """The caller-side variants of the head at the default shape: final RMSNorm inside the call
+    (forward and backward take the un-normalised hidden states) and policy + reference head in one
+    forward launch, each next to the plain call, HIP events, 3 calls each."""
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    dev = torch.device("cuda:0")
+    hidden, weight, targets, grad = make_inputs(torch, cfg, dev)
+    n, h, v = cfg["tokens"], cfg["hidden"], cfg["vocab"]
+    gain = (1.0 + 0.1 * torch.randn(h, device=dev)).to(hidden.dtype)
+    ref_weight = (weight.float() * 1.01).to(weight.dtype)
+    _, lse, _ = LL.fused_linear_logp_forward(hidden, weight, targets)
+    _, lse_n, _ = LL.fused_norm_linear_logp_forward(hidden, gain, weight, targets)
+    out = {
+        "forward_ms": event_ms(torch, lambda: LL.fused_linear_logp_forward(hidden, weight, targets), 3),
+        "forward_with_rmsnorm_ms": event_ms(
+            torch, lambda: LL.fused_norm_linear_logp_forward(hidden, gain, weight, targets), 3),
+        "forward_two_heads_ms": event_ms(
+            torch, lambda: LL.fused_linear_logp_forward_pair(hidden, weight, ref_weight, targets), 3),
+        "backward_ms": event_ms(
+            torch, lambda: LL.fused_linear_logp_backward(grad, hidden, weight, targets, lse), 3),
+        "backward_with_rmsnorm_ms": event_ms(
+            torch, lambda: LL.fused_norm_linear_logp_backward(grad, hidden, gain, weight, targets, lse_n), 3),
+        "note": f"{n} tokens, H={h}, V={v}, {cfg['dtype']}; with_rmsnorm: the call takes the "
+                "un-normalised hidden states and the norm gain (normalised rows only in workspace, "
+                "d_x and d_gain returned); two_heads: policy and reference head in one launch "
+                "(twice the contraction work of forward_ms)",
+    }
+    return out
+
+
 def bench_reference_shapes(torch):
     """The reference's own benchmark shapes and method (benchmarks/benchmark_linear_logp.py:62-86:
     bf16, hidden ~ N(0,1), weight ~ N(0,1), warm-up 5, 20 iterations between device events),
@@ -591,6 +622,8 @@ def main() -> int:
             extras[name]["forward_tflops"] = r["kernels"][0]["achieved"]
             extras[name]["steps"] = 3
             torch.cuda.empty_cache()
+        extras["llama3-8b-head-variants"] = bench_variants(torch, dict(WORKLOADS["llama3-8b-head"]))
+        torch.cuda.empty_cache()
         r = bench_scan(torch, 10, 2, dict(WORKLOADS["logits-scan"]))
         extras["logits-scan"] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "config",
                                                    "bitwise_repeatable", "roofline")}

@@ -159,6 +159,58 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                         int64_t ignore_index, int32_t use_ignore, rlk_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------ *
+ * Final RMSNorm in front of the head (the step before the path).
+ *
+ * rlk_rmsnorm_fwd stands in for NativeRMSNormOp.forward
+ * (rl_engine/kernels/ops/pytorch/norm/rms_norm.py:28-70):
+ *   out = cast_to_dtype( (x * rsqrt(mean(x^2, -1) + eps)) * gain ),  fp32 arithmetic,
+ * x / out [N, H] and gain [H] of `dtype` (bf16 / f16 / f32), rstd [N] f32 optional.  A row's
+ * result does not depend on the other rows of the batch.  rlk_rmsnorm_bwd is its backward
+ * (what autograd derives for that expression): d_x [N, H] of `dtype`, d_gain [H] f32
+ * (overwritten; NULL to skip) from d_out [N, H] of `dtype`; the row statistics are recomputed.
+ * ------------------------------------------------------------------------------------------ */
+int rlk_rmsnorm_fwd(const void* x, const void* gain, float eps, void* out, float* rstd, int64_t N,
+                    int32_t H, int32_t dtype, rlk_stream_t stream);
+
+int rlk_rmsnorm_bwd_workspace_bytes(int64_t N, int32_t H, size_t* bytes);
+
+int rlk_rmsnorm_bwd(const void* x, const void* gain, float eps, const void* d_out, void* d_x,
+                    float* d_gain, void* workspace, size_t workspace_bytes, int64_t N, int32_t H,
+                    int32_t dtype, rlk_stream_t stream);
+
+/* Norm and head as one call each way (no counterpart as a single function in the reference, which
+ * runs the model's final norm and `linear_logp` as separate modules): the entry points take the
+ * UN-normalised hidden states x and the norm gain.
+ *   forward : logp / lse of  linear_logp( rmsnorm(x, gain, eps), weight, bias, ... ),
+ *             bit for bit what rlk_rmsnorm_fwd followed by rlk_linear_logp_fwd return on the same
+ *             blocks of 32768 tokens (the whole input when N <= 32768);
+ *   backward: d_x (gradient w.r.t. the un-normalised hidden states, `dtype`), d_gain [H] f32,
+ *             d_weight [V, H] f32, d_bias [V] f32 -- rlk_linear_logp_bwd followed by rlk_rmsnorm_bwd.
+ * The normalised rows are never saved: they exist as one block of at most 32768 tokens inside the
+ * workspace in either direction (the backward recomputes them), so the caller keeps only x, and the
+ * extra memory stays independent of N.  Any gradient pointer may be NULL. */
+int rlk_linear_logp_rmsnorm_fwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                                                size_t* bytes);
+
+int rlk_linear_logp_rmsnorm_fwd(const void* x, const void* gain, float eps, const void* weight,
+                                const float* bias, const int64_t* targets, float* logp, float* lse,
+                                void* workspace, size_t workspace_bytes, int64_t N, int32_t H,
+                                int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                                int64_t ignore_index, int32_t use_ignore, int32_t strict_targets,
+                                int32_t* err_flag, rlk_stream_t stream);
+
+int rlk_linear_logp_rmsnorm_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
+                                                size_t dz_budget_bytes, size_t* bytes);
+
+int rlk_linear_logp_rmsnorm_bwd(const float* grad_logp, const void* x, const void* gain, float eps,
+                                const void* weight, const float* bias, const int64_t* targets,
+                                const float* lse, void* d_x, float* d_gain, float* d_weight,
+                                float* d_bias, void* workspace, size_t workspace_bytes,
+                                size_t dz_budget_bytes, int64_t N, int32_t H, int64_t V,
+                                int64_t vocab_start, int32_t dtype, float temperature,
+                                int64_t ignore_index, int32_t use_ignore, rlk_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------ *
  * Selected-token log-prob from materialised logits (the `fused_logp` family).
  *
  * Stands in for the nine `_C.fused_logp*` symbols (csrc/ops.cpp:75-96, csrc/fused_logp_kernel.cu:

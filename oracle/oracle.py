@@ -25,6 +25,13 @@ How each function is pinned (see tests/test_oracle_*.py):
                                [-1,1,(x-20)/sqrt(200/3)] (tests/test_grpo_loss.py:110-117).
 * ``grpo_loss_from_logp``      closed-form gradient vs torch autograd of the composition;
                                invariants of tests/test_ratio_kl.py:82-97,163-176.
+* ``rms_norm``                 torch's own ``F.rms_norm`` (independent implementation, 1e-6) and the
+                               hand-written fp32 formula bit for bit, batch-slice invariance
+                               (tests/test_rms_norm.py:22-64 of the reference); unit-gain rows have
+                               mean square 1; scaling x by a power of two leaves the output unchanged
+                               up to eps.
+* ``rms_norm_backward``        torch autograd of ``rms_norm`` in float64; d_x is orthogonal to x
+                               when the gain is 1 and eps is 0 (the norm is scale-invariant).
 """
 
 from __future__ import annotations
@@ -349,3 +356,36 @@ def grpo_loss_from_logp(
     dkl = 1.0 - torch.exp(d)
     grad = torch.where(m, (dpol + beta * dkl) / denom, torch.zeros_like(cur))
     return loss, policy_loss, kl, grad
+
+
+# --------------------------------------------------------------------------- #
+# RMSNorm in front of the head
+# --------------------------------------------------------------------------- #
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, *, eps: float = 1e-6,
+             output_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``x * rsqrt(mean(x^2, -1) + eps) * weight`` accumulated in fp32, cast to ``x.dtype``
+    (or ``output_dtype``).  Follows rl_engine/kernels/ops/pytorch/norm/rms_norm.py:54-70,
+    including its ValueError for a weight that is not ``[x.shape[-1]]``."""
+    if weight.dim() != 1 or weight.shape[0] != x.shape[-1]:
+        raise ValueError(f"weight must be 1-D of size x.shape[-1]={x.shape[-1]}, "
+                         f"got tuple(weight.shape)={tuple(weight.shape)}")
+    x_f = x.float()
+    var = x_f.pow(2).mean(dim=-1, keepdim=True)
+    normed = x_f * torch.rsqrt(var + eps)
+    out = normed * weight.float()
+    return out.to(x.dtype if output_dtype is None else output_dtype)
+
+
+def rms_norm_backward(grad_out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, *,
+                      eps: float = 1e-6) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp32 ``(d_x, d_weight)`` of ``sum(grad_out * rms_norm(x, weight))``: what autograd derives
+    for rl_engine/kernels/ops/pytorch/norm/rms_norm.py:66-70.  With r = rsqrt(mean(x^2) + eps)
+    and g = grad_out * weight:  d_x = r g - x r^3 mean(g x),  d_weight = sum_rows grad_out x r."""
+    x_f = x.float().reshape(-1, x.shape[-1])
+    go = grad_out.float().reshape(-1, x.shape[-1])
+    w = weight.float()
+    r = torch.rsqrt(x_f.pow(2).mean(dim=-1, keepdim=True) + eps)
+    g = go * w
+    d_x = r * g - x_f * r.pow(3) * (g * x_f).mean(dim=-1, keepdim=True)
+    d_w = (go * x_f * r).sum(dim=0)
+    return d_x.reshape(x.shape), d_w

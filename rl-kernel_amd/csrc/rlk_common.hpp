@@ -34,4 +34,13 @@ int generic_bwd(const float* grad_logp, const void* hidden, const void* weight, 
                 float* d_bias, void* workspace, int64_t N, int32_t H, int64_t V,
                 int64_t vocab_start, int32_t dtype, float temperature, int64_t ignore_index,
                 int32_t use_ignore, hipStream_t stream);
+// rlk_linear_logp_bwd with one more switch: accumulate != 0 adds d_weight / d_bias to what the
+// buffers already hold (callers that feed the tokens in several blocks).
+int linear_logp_bwd_accumulating(const float* grad_logp, const void* hidden, const void* weight,
+                                 const float* bias, const int64_t* targets, const float* lse,
+                                 void* d_hidden, float* d_weight, float* d_bias, void* workspace,
+                                 size_t workspace_bytes, size_t dz_budget_bytes, int64_t N, int32_t H,
+                                 int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                                 int64_t ignore_index, int32_t use_ignore, int32_t accumulate,
+                                 hipStream_t stream);
 }  // namespace rlk

@@ -1231,6 +1231,7 @@ struct BwdCall {
     int64_t ignore_index;
     int32_t use_ignore;
     hipStream_t stream;
+    int accumulate;  // 1: d_weight / d_bias already hold the sums of earlier tokens, add to them
 };
 
 // Grid of a chained launch: one workgroup per compute unit, rounded down to a multiple of 8 so
@@ -1336,7 +1337,7 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             d.tok_valid = tok_valid;
             d.v_tiles = v_tiles;
             d.h_tiles = h_tiles;
-            d.accumulate = ci > 0;
+            d.accumulate = ci > 0 || c.accumulate != 0;
 
             // dZ block: full vocab tiles through the fast variant (chained through one pipeline
             // when the token tiles are full too), the rest (all of them when there is a bias)
@@ -1394,7 +1395,7 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             if (c.d_bias != nullptr) {
                 hipLaunchKernelGGL(linear_logp_db_kernel, dim3((v_valid + 255) / 256), dim3(256), 0,
                                    stream, dz, p.ldz, tok_valid, v_valid, scales, c.d_bias + v_lo,
-                                   ci > 0 ? 1 : 0, c.dtype);
+                                   (ci > 0 || c.accumulate != 0) ? 1 : 0, c.dtype);
             }
             if (int rc = check_launch("linear_logp backward launch failed")) return rc;
         }
@@ -1772,6 +1773,22 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                         int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
                         int64_t ignore_index, int32_t use_ignore, hipStream_t stream)
 {
+    return rlk::linear_logp_bwd_accumulating(grad_logp, hidden, weight, bias, targets, lse, d_hidden,
+                                             d_weight, d_bias, workspace, workspace_bytes,
+                                             dz_budget_bytes, N, H, V, vocab_start, dtype, temperature,
+                                             ignore_index, use_ignore, 0, stream);
+}
+
+}  // extern "C"
+
+int rlk::linear_logp_bwd_accumulating(const float* grad_logp, const void* hidden, const void* weight,
+                                      const float* bias, const int64_t* targets, const float* lse,
+                                      void* d_hidden, float* d_weight, float* d_bias, void* workspace,
+                                      size_t workspace_bytes, size_t dz_budget_bytes, int64_t N,
+                                      int32_t H, int64_t V, int64_t vocab_start, int32_t dtype,
+                                      float temperature, int64_t ignore_index, int32_t use_ignore,
+                                      int32_t accumulate, hipStream_t stream)
+{
     if (int rc = check_common(N, H, V, dtype)) return rc;
     if (!(temperature > 0.f)) return rlk_fail(RLK_ERR_ARG, "temperature must be greater than zero");
     if (!grad_logp || !hidden || !weight || !targets || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
@@ -1783,16 +1800,17 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
     if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
     if (reinterpret_cast<uintptr_t>(workspace) & 255)
         return rlk_fail(RLK_ERR_ARG, "workspace must be 256-byte aligned");
-    if (!use_mfma(hidden, weight, H, dtype))
+    if (!use_mfma(hidden, weight, H, dtype)) {
+        if (accumulate && (d_weight || d_bias))
+            return rlk_fail(RLK_ERR_UNSUPPORTED, "the scalar path cannot add to existing gradients");
         return generic_bwd(grad_logp, hidden, weight, bias, targets, lse, d_hidden, d_weight, d_bias,
                            workspace, N, H, V, vocab_start, dtype, temperature, ignore_index,
                            use_ignore, stream);
+    }
     const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
     int n_cu = 0;
     if (int rc = compute_units(&n_cu)) return rc;
     BwdCall c{grad_logp, hidden, weight, bias, targets, lse, d_hidden, d_weight, d_bias, workspace,
-              N, H, V, vocab_start, dtype, temperature, ignore_index, use_ignore, stream};
+              N, H, V, vocab_start, dtype, temperature, ignore_index, use_ignore, stream, accumulate};
     return dtype == RLK_DTYPE_BF16 ? bwd_enqueue<Bf16>(c, p, n_cu) : bwd_enqueue<F16>(c, p, n_cu);
 }
-
-}  // extern "C"

@@ -164,6 +164,91 @@ def fused_linear_logp_forward_pair(
     return (*outs, err)
 
 
+def fused_norm_linear_logp_forward(
+    x_2d: torch.Tensor,
+    gain: torch.Tensor,
+    weight: torch.Tensor,
+    target_1d: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    *,
+    eps: float = 1e-6,
+    temperature: float = 1.0,
+    ignore_index: Optional[int] = None,
+):
+    """Raw forward from UN-normalised hidden states: ``(logp, lse, err_flag)`` of
+    ``linear_logp(rmsnorm(x, gain, eps), weight, bias)``; the normalised rows live only in the
+    call's workspace."""
+    lib = _native.load()
+    n, h = x_2d.shape
+    v = weight.size(0)
+    dev = x_2d.device
+    logp = torch.empty(n, device=dev, dtype=torch.float32)
+    lse = torch.empty(n, device=dev, dtype=torch.float32)
+    err = torch.zeros(1, device=dev, dtype=torch.int32)
+    if n == 0:
+        return logp, lse, err
+    _warn_if_scalar_path(x_2d, weight)
+    need = _native.ctypes.c_size_t(0)
+    dt = _DTYPES[x_2d.dtype]
+    _native.check(lib.rlk_linear_logp_rmsnorm_fwd_workspace_bytes(n, h, v, dt, _native.ctypes.byref(need)),
+                  "norm + linear_logp workspace query")
+    ws = torch.empty(max(need.value, 256), device=dev, dtype=torch.uint8)
+    bias_f = None if bias is None else bias.detach().to(torch.float32).contiguous()
+    rc = lib.rlk_linear_logp_rmsnorm_fwd(
+        _ptr(x_2d), _ptr(gain), float(eps), _ptr(weight), _ptr(bias_f), _ptr(target_1d), _ptr(logp),
+        _ptr(lse), _ptr(ws), ws.numel(), n, h, v, 0, dt, float(temperature),
+        0 if ignore_index is None else int(ignore_index), int(ignore_index is not None), 1,
+        _ptr(err), _stream(dev))
+    _native.check(rc, "rlk_linear_logp_rmsnorm_fwd")
+    return logp, lse, err
+
+
+def fused_norm_linear_logp_backward(
+    grad_logp: torch.Tensor,
+    x_2d: torch.Tensor,
+    gain: torch.Tensor,
+    weight: torch.Tensor,
+    target_1d: torch.Tensor,
+    lse: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    *,
+    eps: float = 1e-6,
+    temperature: float = 1.0,
+    ignore_index: Optional[int] = None,
+    need_x: bool = True,
+    need_gain: bool = True,
+    need_weight: bool = True,
+    need_bias: bool = True,
+    dz_budget_bytes: int = 0,
+):
+    """Raw backward: ``(d_x [N,H] input dtype, d_gain [H] fp32, d_weight [V,H] fp32, d_bias [V]
+    fp32)``; ``d_x`` is the gradient w.r.t. the UN-normalised hidden states."""
+    lib = _native.load()
+    n, h = x_2d.shape
+    v = weight.size(0)
+    dev = x_2d.device
+    dt = _DTYPES[x_2d.dtype]
+    g = grad_logp.reshape(-1).to(torch.float32).contiguous()
+    d_x = torch.empty_like(x_2d) if need_x else None
+    d_gain = torch.empty(h, device=dev, dtype=torch.float32) if need_gain else None
+    d_weight = torch.empty(v, h, device=dev, dtype=torch.float32) if need_weight else None
+    want_bias = bias is not None and need_bias
+    d_bias = torch.empty(v, device=dev, dtype=torch.float32) if want_bias else None
+    bias_f = None if bias is None else bias.detach().to(torch.float32).contiguous()
+    need = _native.ctypes.c_size_t(0)
+    _native.check(lib.rlk_linear_logp_rmsnorm_bwd_workspace_bytes(n, h, v, dt, int(dz_budget_bytes),
+                                                                  _native.ctypes.byref(need)),
+                  "norm + linear_logp backward workspace query")
+    ws = torch.empty(max(need.value, 256), device=dev, dtype=torch.uint8)
+    rc = lib.rlk_linear_logp_rmsnorm_bwd(
+        _ptr(g), _ptr(x_2d), _ptr(gain), float(eps), _ptr(weight), _ptr(bias_f), _ptr(target_1d),
+        _ptr(lse), _ptr(d_x), _ptr(d_gain), _ptr(d_weight), _ptr(d_bias), _ptr(ws), ws.numel(),
+        int(dz_budget_bytes), n, h, v, 0, dt, float(temperature),
+        0 if ignore_index is None else int(ignore_index), int(ignore_index is not None), _stream(dev))
+    _native.check(rc, "rlk_linear_logp_rmsnorm_bwd")
+    return d_x, d_gain, d_weight, d_bias
+
+
 def fused_linear_logp_backward(
     grad_logp: torch.Tensor,
     hidden_2d: torch.Tensor,
@@ -260,6 +345,51 @@ class _FusedLinearLogpFunction(torch.autograd.Function):
         return grad_hidden, grad_weight, grad_bias, None, None, None, None
 
 
+class _FusedNormLinearLogpFunction(torch.autograd.Function):
+    """linear_logp(rmsnorm(x, gain)) from the un-normalised hidden states; saves x, not the
+    normalised rows."""
+
+    @staticmethod
+    def forward(ctx, x, gain, weight, bias, target_ids, eps, temperature, ignore_index, check_targets):
+        x_2d = _aligned_contiguous(x.reshape(-1, x.size(-1)))
+        g = _aligned_contiguous(gain.to(x.dtype))
+        w = _aligned_contiguous(weight)
+        target_1d = target_ids.reshape(-1).to(device=x_2d.device, dtype=torch.long).contiguous()
+        logp, lse, err = fused_norm_linear_logp_forward(
+            x_2d, g, w, target_1d, bias, eps=eps, temperature=temperature, ignore_index=ignore_index)
+        ctx.empty = x_2d.size(0) == 0
+        if check_targets and not ctx.empty and bool(err.item()):
+            raise _out_of_range_error(target_1d, w.size(0), ignore_index)
+        ctx.save_for_backward(x_2d, g, w, bias if bias is not None else x_2d, target_1d, lse)
+        ctx.has_bias = bias is not None
+        ctx.lead_shape = x.shape[:-1]
+        ctx.eps, ctx.temperature, ctx.ignore_index = eps, temperature, ignore_index
+        ctx.gain_dtype, ctx.weight_dtype = gain.dtype, weight.dtype
+        ctx.bias_dtype = bias.dtype if bias is not None else None
+        return logp.reshape(x.shape[:-1])
+
+    @staticmethod
+    def backward(ctx, grad_logp):
+        x_2d, g, w, bias_t, target_1d, lse = ctx.saved_tensors
+        need_x, need_g, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
+        need_b = ctx.has_bias and ctx.needs_input_grad[3]
+        if ctx.empty:
+            return (torch.zeros(tuple(ctx.lead_shape) + (x_2d.size(1),), device=x_2d.device,
+                                dtype=x_2d.dtype) if need_x else None,
+                    torch.zeros_like(g, dtype=ctx.gain_dtype) if need_g else None,
+                    torch.zeros_like(w, dtype=ctx.weight_dtype) if need_w else None,
+                    torch.zeros_like(bias_t, dtype=ctx.bias_dtype) if need_b else None,
+                    None, None, None, None, None)
+        d_x, d_g, d_w, d_b = fused_norm_linear_logp_backward(
+            grad_logp, x_2d, g, w, target_1d, lse, bias_t if ctx.has_bias else None, eps=ctx.eps,
+            temperature=ctx.temperature, ignore_index=ctx.ignore_index, need_x=need_x,
+            need_gain=need_g, need_weight=need_w, need_bias=need_b)
+        return (d_x.reshape(tuple(ctx.lead_shape) + (x_2d.size(1),)) if need_x else None,
+                d_g.to(ctx.gain_dtype) if need_g else None,
+                d_w.to(ctx.weight_dtype) if need_w else None,
+                d_b.to(ctx.bias_dtype) if need_b else None, None, None, None, None, None)
+
+
 class _FusedLinearLogpPairFunction(torch.autograd.Function):
     """Policy log-probs (differentiable) and reference log-probs (no gradient) from one launch."""
 
@@ -308,17 +438,25 @@ class RocmFusedLinearLogpOp:
     def __call__(self, hidden, lm_head_weight, target_ids, bias=None, *, tp_group: Any = None,
                  vocab_start_index: int = 0, global_vocab_size: Optional[int] = None,
                  temperature: float = 1.0, ignore_index: Optional[int] = None,
-                 check_targets: bool = True) -> torch.Tensor:
+                 check_targets: bool = True, norm_weight: Optional[torch.Tensor] = None,
+                 norm_eps: float = 1e-6) -> torch.Tensor:
         return self.apply(hidden, lm_head_weight, target_ids, bias, tp_group=tp_group,
                           vocab_start_index=vocab_start_index, global_vocab_size=global_vocab_size,
                           temperature=temperature, ignore_index=ignore_index,
-                          check_targets=check_targets)
+                          check_targets=check_targets, norm_weight=norm_weight, norm_eps=norm_eps)
 
     def apply(self, hidden, lm_head_weight, target_ids, bias=None, *, tp_group: Any = None,
               vocab_start_index: int = 0, global_vocab_size: Optional[int] = None,
               temperature: float = 1.0, ignore_index: Optional[int] = None,
-              check_targets: bool = True) -> torch.Tensor:
-        """Selected-token log-prob in float32 with the leading shape of ``hidden``."""
+              check_targets: bool = True, norm_weight: Optional[torch.Tensor] = None,
+              norm_eps: float = 1e-6) -> torch.Tensor:
+        """Selected-token log-prob in float32 with the leading shape of ``hidden``.
+
+        ``norm_weight`` (keyword-only, default off): ``hidden`` is then the UN-normalised output
+        of the last layer and the model's final RMSNorm
+        (rl_engine/kernels/ops/pytorch/norm/rms_norm.py:54-70 of the reference, gain
+        ``norm_weight``, ``norm_eps``) runs inside the op; the gradient flows to the un-normalised
+        hidden states and to the gain, and the normalised activations are never kept."""
         if temperature <= 0.0:
             raise ValueError("temperature must be greater than zero")
         if lm_head_weight.size(-1) != hidden.size(-1):
@@ -358,6 +496,16 @@ class RocmFusedLinearLogpOp:
             raise NotImplementedError(
                 "RocmFusedLinearLogpOp needs hidden and lm_head_weight of one dtype "
                 "(bf16, f16 or f32) on the same GPU")
+        if norm_weight is not None:
+            if norm_weight.dim() != 1 or norm_weight.shape[0] != hidden.size(-1):
+                raise ValueError(f"norm_weight must be 1-D of size hidden.shape[-1]={hidden.size(-1)}, "
+                                 f"got tuple(norm_weight.shape)={tuple(norm_weight.shape)}")
+            if norm_weight.device != hidden.device:
+                raise ValueError(f"norm_weight device {norm_weight.device} must match hidden device "
+                                 f"{hidden.device}")
+            return _FusedNormLinearLogpFunction.apply(hidden, norm_weight, lm_head_weight, bias,
+                                                      target_ids, float(norm_eps), float(temperature),
+                                                      ignore_index, check_targets)
         return _FusedLinearLogpFunction.apply(hidden, lm_head_weight, bias, target_ids,
                                               float(temperature), ignore_index, check_targets)
 

@@ -36,6 +36,7 @@ class OpBackend(Enum, metaclass=_KernelEnumMeta):
     ROCM_GRPO_LOSS = "rl_kernel_amd.ops.grpo.RocmGRPOLossOp"
     ROCM_GRPO_FROM_LOGP = "rl_kernel_amd.ops.grpo.RocmGRPOFromLogpOp"
     ROCM_GRPO_STEP = "rl_kernel_amd.ops.grpo_step.RocmFusedGRPOStepOp"
+    ROCM_RMS_NORM = "rl_kernel_amd.ops.rms_norm.RocmRMSNormOp"
 
 
 _LOGP_TYPES = ("logp", "logp_indexed", "logp_online", "logp_online_indexed")
@@ -51,6 +52,7 @@ class KernelRegistry:
             "grpo_loss": [OpBackend.ROCM_GRPO_LOSS],
             "grpo_loss_from_logp": [OpBackend.ROCM_GRPO_FROM_LOGP],
             "grpo_step_from_hidden": [OpBackend.ROCM_GRPO_STEP],
+            "rms_norm": [OpBackend.ROCM_RMS_NORM],
         }
         for name in _LOGP_TYPES:
             rocm[name] = [OpBackend.ROCM_FUSED_LOGP]

@@ -292,3 +292,60 @@ def test_grpo_masked_garbage_invariance_and_gradient_linearity():
     assert torch.allclose(base[3], other[3])
     empty = O.grpo_loss_from_logp(cur, old, ref, adv, torch.zeros_like(mask), beta=0.04)
     assert empty[0].item() == 0.0 and torch.equal(empty[3], torch.zeros_like(cur))
+
+
+# --------------------------------------------------------------------------- #
+# RMSNorm (the step in front of the head)
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("n", [4096, 128])
+def test_rms_norm_matches_torch_rms_norm_and_the_manual_formula(n):
+    """tests/test_rms_norm.py:22-49 of the reference: torch's own F.rms_norm is an independent
+    implementation (tolerance, the reduction order may differ); the hand-written fp32 formula in
+    the same float order must agree bit for bit."""
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2, 16, n, generator=g)
+    w = torch.randn(n, generator=torch.Generator().manual_seed(1))
+    got = O.rms_norm(x, w, output_dtype=torch.float32)
+    torch.testing.assert_close(got, F.rms_norm(x, (n,), weight=w, eps=1e-6), rtol=1e-6, atol=1e-6)
+    x_f = x.float()
+    manual = x_f * torch.rsqrt(x_f.pow(2).mean(dim=-1, keepdim=True) + 1e-6) * w.float()
+    assert torch.equal(got, manual)
+    # a row's output does not depend on how many rows share the batch (same file :55-64)
+    assert torch.equal(O.rms_norm(x[:1], w, output_dtype=torch.float32), got[:1])
+    assert torch.equal(O.rms_norm(x[1:, 3:5], w, output_dtype=torch.float32), got[1:, 3:5])
+
+
+def test_rms_norm_closed_form_properties_and_dtype_policy():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(5, 64, generator=g) * 3.0
+    ones = torch.ones(64)
+    out = O.rms_norm(x, ones, eps=0.0)
+    assert torch.allclose(out.pow(2).mean(dim=-1), torch.ones(5), atol=1e-5)      # unit mean square
+    assert torch.allclose(O.rms_norm(4.0 * x, ones, eps=0.0), out, atol=1e-6)    # scale invariance
+    # known answer: x = [3, 4] -> mean square 12.5 -> [3, 4] / sqrt(12.5) times the gain
+    ka = O.rms_norm(torch.tensor([[3.0, 4.0]]), torch.tensor([2.0, 0.5]), eps=0.0)
+    assert torch.allclose(ka, torch.tensor([[6.0, 2.0]]) / 12.5 ** 0.5, atol=1e-6)
+    # the result is computed in fp32 and cast once to the input dtype
+    xb = x.to(torch.bfloat16)
+    wb = torch.randn(64, generator=g).to(torch.bfloat16)
+    assert O.rms_norm(xb, wb).dtype == torch.bfloat16
+    assert torch.equal(O.rms_norm(xb, wb), O.rms_norm(xb, wb, output_dtype=torch.float32).to(torch.bfloat16))
+    with pytest.raises(ValueError, match="weight must be 1-D"):
+        O.rms_norm(x, torch.ones(63))
+
+
+def test_rms_norm_backward_matches_autograd():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(7, 48, generator=g, dtype=torch.float64).requires_grad_(True)
+    w = torch.randn(48, generator=g, dtype=torch.float64).requires_grad_(True)
+    go = torch.randn(7, 48, generator=g, dtype=torch.float64)
+    y = x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + 1e-6) * w     # float64 autograd
+    (y * go).sum().backward()
+    d_x, d_w = O.rms_norm_backward(go.float(), x.detach().float(), w.detach().float())
+    assert torch.allclose(d_x.double(), x.grad, atol=1e-5)
+    assert torch.allclose(d_w.double(), w.grad, atol=1e-5)
+    # scale invariance of the norm: with unit gain and eps = 0 the gradient is orthogonal to x
+    d_x0, _ = O.rms_norm_backward(go.float(), x.detach().float(), torch.ones(48), eps=0.0)
+    assert (d_x0 * x.detach().float()).sum(dim=-1).abs().max().item() < 1e-4
