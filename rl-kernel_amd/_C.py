@@ -1,10 +1,16 @@
 """Native symbol table of the gfx950 backend, under the names the reference's compiled module
 exposes (csrc/ops.cpp:75-99, rl_engine/_C.pyi:5-43 of the reference) so that wrappers probing
 ``hasattr(_C, name)`` find them.  ``fused_linear_logp`` is the device-neutral name of what the
-reference calls ``fused_linear_logp_sm90``; both names are bound."""
+reference calls ``fused_linear_logp_sm90``; both names are bound.
+
+Two routes to the same C ABI: the compiled PyTorch extension ``lib/_rlk_C.so`` (pybind11, built by
+``build.py`` from ``csrc/rlk_torch_binding.cpp``) when it is there, otherwise the ctypes wrappers
+below.  ``COMPILED`` says which one is bound."""
 
 from __future__ import annotations
 
+import importlib.util
+import os
 from typing import List, Optional
 
 import torch
@@ -71,3 +77,24 @@ def fused_linear_logp(hidden: torch.Tensor, weight: torch.Tensor, target: torch.
 
 
 fused_linear_logp_sm90 = fused_linear_logp
+
+
+
+def _load_compiled():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "_rlk_C.so")
+    if not os.path.exists(path):
+        return None
+    spec = importlib.util.spec_from_file_location("_rlk_C", path)
+    module = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(module)
+    return module
+
+
+_PYTHON_ROUTE = {name: obj for name, obj in list(globals().items())
+                 if name.startswith("fused_") and callable(obj)}
+compiled_module = _load_compiled()
+COMPILED = compiled_module is not None
+if COMPILED:
+    for _name in _PYTHON_ROUTE:
+        if hasattr(compiled_module, _name):
+            globals()[_name] = getattr(compiled_module, _name)

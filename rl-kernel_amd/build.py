@@ -44,6 +44,36 @@ def _check_no_packed_fp32(asm_path: str, src: str) -> None:
                            f"({len(hits)}, first: {hits[0]}); the -packed-fp32-ops switch did not take effect")
 
 
+BINDING_SRC = "rlk_torch_binding.cpp"
+BINDING_NAME = "_rlk_C"
+BINDING_PATH = os.path.join(LIB_DIR, BINDING_NAME + ".so")
+
+
+def _binding_compile_cmd(obj: str):
+    """hipcc line that compiles the PyTorch binding (host code, torch + pybind11 headers)."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    incs = [os.path.join(os.path.dirname(HERE), "include"), *ce.include_paths("cuda"),
+            sysconfig.get_paths()["include"]]
+    abi = int(bool(getattr(torch._C, "_GLIBCXX_USE_CXX11_ABI", True)))
+    return [hipcc(), "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-x", "hip", "-c",
+            os.path.join(CSRC, BINDING_SRC), "-o", obj, f"-DTORCH_EXTENSION_NAME={BINDING_NAME}",
+            "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_API_INCLUDE_EXTENSION_H",
+            f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-Wno-unused-result", *[f"-I{i}" for i in incs]]
+
+
+def _binding_link_cmd(obj: str, out: str):
+    from torch.utils import cpp_extension as ce
+
+    torch_lib = ce.library_paths()[0]
+    return [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", obj, "-o", out, f"-L{torch_lib}",
+            "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+            f"-L{LIB_DIR}", "-lrlk_hip", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+
+
 def build(verbose: bool = False, extra_flags=()) -> str:
     """Compile every source and link the shared library. Always recompiles.  Every source is
     also compiled to device assembly once more to verify that no packed-fp32 instruction was
@@ -64,6 +94,11 @@ def build(verbose: bool = False, extra_flags=()) -> str:
         procs.append((src, None, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
         procs.append((src, asm, subprocess.Popen(chk, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
         objs.append(obj)
+    # the compiled PyTorch binding (the reference's `_C` symbol names over this C ABI): its
+    # compile runs beside the kernels', its link needs the library
+    bind_obj = os.path.join(LIB_DIR, BINDING_NAME + ".o")
+    bind_proc = subprocess.Popen(_binding_compile_cmd(bind_obj), stdout=subprocess.PIPE,
+                                 stderr=subprocess.STDOUT)
     for src, asm, proc in procs:
         out = proc.communicate()[0].decode()
         if proc.returncode != 0:
@@ -79,8 +114,19 @@ def build(verbose: bool = False, extra_flags=()) -> str:
     if res.returncode != 0:
         raise RuntimeError("link failed:\n" + res.stdout.decode())
     os.replace(tmp, LIB_PATH)
+    out = bind_proc.communicate()[0].decode()
+    if bind_proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {BINDING_SRC}:\n{out}")
+    tmp = BINDING_PATH + ".tmp"
+    res = subprocess.run(_binding_link_cmd(bind_obj, tmp), stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    if res.returncode != 0:
+        raise RuntimeError("link of the PyTorch binding failed:\n" + res.stdout.decode())
+    os.replace(tmp, BINDING_PATH)
     return LIB_PATH
 
 
 if __name__ == "__main__":
+    # run as a script, this directory heads sys.path and its platform.py would shadow the standard
+    # library's `platform` for every later import (torch's included)
+    sys.path = [p for p in sys.path if os.path.abspath(p or ".") != HERE]
     print(build(verbose="-v" in sys.argv))

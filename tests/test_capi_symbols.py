@@ -158,3 +158,24 @@ def test_backward_plan_keeps_in_tile_offsets_within_32_bits(native, n, h, v, bud
     need = ctypes.c_size_t(0)
     assert lib.rlk_linear_logp_bwd_workspace_bytes(n, h, v, 0, budget, ctypes.byref(need)) == 0
     assert need.value <= (3 << 30) + (1 << 20)          # block + fp32 dH chunk <= 1.5 x 2 GiB
+
+
+def test_compiled_pytorch_binding_exports_the_reference_symbol_names(native):
+    """The pybind11 extension built from csrc/rlk_torch_binding.cpp carries the names the
+    reference registers in csrc/ops.cpp:75-99 (all but the attention op, which is off this path),
+    and rl_kernel_amd._C binds them in place of its ctypes route."""
+    from rl_kernel_amd import _C
+
+    assert os.path.exists(os.path.join(os.path.dirname(native.LIB_PATH), "_rlk_C.so"))
+    assert _C.COMPILED
+    names = ["fused_logp", "fused_logp_sm90", "fused_linear_logp_sm90", "fused_logp_forward_out",
+             "fused_logp_forward_fp32", "fused_logp_forward_indexed_out",
+             "fused_logp_forward_indexed_fp32", "fused_logp_forward_online_out",
+             "fused_logp_forward_online_fp32", "fused_logp_forward_online_indexed_out",
+             "fused_logp_forward_online_indexed_fp32"]
+    for name in names:
+        assert hasattr(_C.compiled_module, name), name
+    for name in names:
+        if name != "fused_logp_sm90":
+            assert getattr(_C, name) is getattr(_C.compiled_module, name), name
+    assert _C.compiled_module.rlk_version() == native.load().rlk_version()

@@ -140,3 +140,45 @@ def test_full_vocab_rows_property(dev, op):
         lp = op.apply_fp32(rep, chunk.repeat(4))
         total += lp.double().exp().view(4, -1).sum(1)
     assert torch.allclose(total, torch.ones(4, device=dev, dtype=torch.float64), atol=1e-4)
+
+
+def test_compiled_binding_calls_reach_the_kernels(dev):
+    """`fused_linear_logp_sm90` and the `fused_logp_forward_*` family through the compiled PyTorch
+    extension (the names of csrc/ops.cpp:75-99 of the reference): values against the oracle,
+    storage identity of the `*_out` forms, RuntimeError for malformed arguments."""
+    from rl_kernel_amd import _C
+
+    assert _C.COMPILED
+    mod = _C.compiled_module
+    g = torch.Generator().manual_seed(17)
+    hidden = torch.randn(300, 128, generator=g).to(torch.bfloat16)
+    weight = (torch.randn(1000, 128, generator=g) * 0.1).to(torch.bfloat16)
+    bias = torch.randn(1000, generator=g) * 0.2
+    target = torch.randint(0, 1000, (300,), generator=g)
+    logp, lse = mod.fused_linear_logp_sm90(hidden.to(dev), weight.to(dev), target.to(dev).int(),
+                                           bias.to(dev))
+    want, want_lse = O.linear_logp(hidden, weight, target, bias, return_lse=True)
+    assert logp.dtype == torch.float32 and (logp.cpu() - want).abs().max().item() < 1e-3
+    assert (lse.cpu() - want_lse).abs().max().item() < 1e-3
+    no_bias = mod.fused_linear_logp_sm90(hidden.to(dev), weight.to(dev), target.to(dev))
+    assert (no_bias[0].cpu() - O.linear_logp(hidden, weight, target)).abs().max().item() < 1e-3
+    # a vocab shard: targets outside it report logp = -lse
+    shard = mod.fused_linear_logp(hidden.to(dev), weight[:500].contiguous().to(dev), target.to(dev), None)
+    outside = (target >= 500).to(dev)
+    assert torch.equal(shard[0][outside], -shard[1][outside])
+    with pytest.raises(RuntimeError, match="hidden-dim mismatch"):
+        mod.fused_linear_logp_sm90(hidden.to(dev), weight[:, :64].contiguous().to(dev), target.to(dev))
+
+    logits = (torch.randn(50, 777, generator=g) * 2).to(torch.float16).to(dev)
+    ids = torch.randint(0, 777, (50,), generator=g).to(dev)
+    out = torch.full((50,), 123.0, device=dev)
+    ret = mod.fused_logp_forward_out(logits, ids, out)
+    assert ret.data_ptr() == out.data_ptr()
+    ref = O.logp_from_logits(logits.cpu(), ids.cpu())
+    assert (out.cpu() - ref).abs().max().item() < 2e-3
+    rows = torch.tensor([3, 7, 49], device=dev)
+    part = mod.fused_logp_forward_online_indexed_fp32(logits, ids, rows)
+    assert torch.equal(part[rows], out[rows]) and part.sum().item() == out[rows].sum().item()
+    assert mod.fused_logp(logits, ids).dtype == torch.float16
+    with pytest.raises(RuntimeError, match="token_ids must be int64"):
+        mod.fused_logp_forward_fp32(logits, ids.int())
