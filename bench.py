@@ -43,8 +43,15 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "",
-    "bytes_per_launch": {},
+    "kernel_source_sha16": "f40ed3feaf6d5501",
+    "measured_at_commit": "32aaa94",
+    "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
+    "bytes_per_launch": {
+        "linear_logp_fwd_kernel": 51445453564,
+        "linear_logp_dz_kernel": 1963404015,
+        "linear_logp_dh_kernel": 1837065263,
+        "linear_logp_dw_kernel": 2158194980,
+    },
 }
 
 WORKLOADS = {
@@ -216,7 +223,8 @@ def bwd_plan(n, h, v, dtype_id):
     return dict(tok_chunk=out[0], v_piece=out[1], n_chunks=out[2], n_pieces=out[3], dh_parts=out[4])
 
 
-def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False):
+def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False, registry_op=False,
+                 probe_epilogue=True):
     """Forward(+backward) of the fused LM-head logp through the raw C-ABI wrappers."""
     from rl_kernel_amd.ops import linear_logp as LL
 
@@ -315,6 +323,8 @@ def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False
         "bitwise_repeatable": bool(deterministic),
     }
     if grpo:
+        res["metric"] = "GRPO step (logp fwd + loss epilogue + bwd) tokens/sec"
+    if grpo and probe_epilogue:
         # The loss epilogue rides in the forward's last launch.  At the full head its cost drowns
         # in the +-1 % run-to-run spread of the 25 ms contraction, so it is measured where the
         # contraction is negligible: the same 32768 tokens, masks, advantages and log-prob inputs
@@ -360,7 +370,6 @@ def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False
         epi_ms = max(tiny_f - tiny_p, 1e-4)
         del th, tw, tt, adv0
         epi_bytes = n * (4 + 4 + 4 + 1 + 4 + 4)  # cur, old, ref, mask in; d_cur, d_kl out
-        res["metric"] = "GRPO step (logp fwd + loss epilogue + bwd) tokens/sec"
         res["epilogue"] = {
             "bound": "hbm", "ms": epi_ms, "algorithmic_bytes": epi_bytes,
             "full_head_forward_ms": plain, "full_head_forward_with_epilogue_ms": fused,
@@ -417,13 +426,20 @@ def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False
         if name == MEASURED_TRAFFIC["workload"] and sha == MEASURED_TRAFFIC["kernel_source_sha16"]:
             traffic = MEASURED_TRAFFIC["bytes_per_launch"].get(k["kernel"])
         k["traffic"] = traffic
+    if name == MEASURED_TRAFFIC["workload"]:
+        res["traffic_source"] = (
+            f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at commit {MEASURED_TRAFFIC['measured_at_commit']} "
+            f"(kernel sources {MEASURED_TRAFFIC['kernel_source_sha16']}), see profiles/"
+            if sha == MEASURED_TRAFFIC["kernel_source_sha16"] else
+            f"null: the kernel sources ({sha}) differ from the ones the counters were read with "
+            f"({MEASURED_TRAFFIC['kernel_source_sha16']})")
     res["kernels"] = kernels
     res["kernel_source_sha16"] = sha
     dominant = max(kernels, key=lambda k: k["launch_ms"] * k["launches_per_step"])
     res["roofline"] = dict(dominant)
     res["roofline"]["note"] = "the kernel with the largest share of the step; see `kernels` for all four"
 
-    if detailed and do_bwd and not grpo:
+    if registry_op and do_bwd and not grpo:
         res["through_registry_op"] = bench_registry_op(torch, hidden, weight, targets, grad, temp, ign,
                                                        max(2, steps // 4))
     return res
@@ -547,7 +563,8 @@ def main() -> int:
     ap.add_argument("--dtype", default=None, choices=["bf16", "f16"],
                     help="override the workload's 16-bit input type")
     ap.add_argument("--no-extras", action="store_true",
-                    help="skip the extra workloads, the registry-op timing and the vendor GEMM")
+                    help="skip the extra workloads, the registry-op timing, the vendor GEMM and the "
+                         "tiny-head probe of the loss epilogue (what a profiler run wants)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known HBM traffic) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
@@ -589,7 +606,8 @@ def main() -> int:
     main_default = args.workload == "llama3-8b-head" and args.mode == "fwd+bwd" and not args.no_extras
     result = dict(common)
     result.update(bench_linear(torch, args.workload, cfg, args.steps, args.warmup, args.mode,
-                               detailed=not args.no_extras))
+                               detailed=True, registry_op=not args.no_extras,
+                               probe_epilogue=not args.no_extras))
     result["device"] = device_info(torch)
     torch.cuda.empty_cache()
 
