@@ -15,7 +15,7 @@ Prints ONE JSON line.  Besides the headline metric (tokens/s of the whole step) 
     and autograd (adds the target-range check and the cast of dW to the weight dtype);
   * `extra_workloads`: the other benchmark configurations (64k tokens at T=0.7, the Qwen3 head in
     f16 with 1 % ignored positions, the GRPO step with its loss epilogue, the logits-fed scan) and
-    the shapes the reference publishes H100 latencies for, a few steps each;
+    the shapes the reference publishes H100 latencies for, fp32 inputs, a few steps each;
   * `cpu_baseline`: the CPU oracle (F.linear -> log_softmax -> gather in fp32, autograd backward)
     timed on a 2048-token slice on the host cores.
 """
@@ -551,6 +551,38 @@ def bench_reference_shapes(torch):
             "rows": rows}
 
 
+def bench_fp32_inputs(torch):
+    """fp32 hidden states and head (what the reference runs in its CPU tests and what callers that keep
+    an fp32 lm_head pass): the same entry points on the fp32 matrix instruction, priced against the
+    157.3 TFLOP/s fp32 matrix peak; a plain fp32 library GEMM of the forward's shape beside it."""
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    dev = torch.device("cuda:0")
+    rows = []
+    for n, h, v in ((4096, 2048, 32768), (2048, 4096, 128256)):
+        gen = torch.Generator(device=dev).manual_seed(v)
+        hidden = torch.randn(n, h, device=dev, generator=gen)
+        weight = torch.randn(v, h, device=dev, generator=gen) * 0.02
+        target = torch.randint(0, v, (n,), device=dev, generator=gen)
+        grad = torch.randn(n, device=dev, generator=gen)
+        _, lse, _ = LL.fused_linear_logp_forward(hidden, weight, target)
+        fwd = lambda: LL.fused_linear_logp_forward(hidden, weight, target)
+        bwd = lambda: LL.fused_linear_logp_backward(grad, hidden, weight, target, lse)
+        gemm = lambda: torch.matmul(hidden, weight.t())
+        for f in (fwd, bwd, gemm):
+            f()
+        f_ms, b_ms, g_ms = event_ms(torch, fwd, 5), event_ms(torch, bwd, 3), event_ms(torch, gemm, 5)
+        flop = 2.0 * n * h * v
+        rows.append({"shape": f"{n}x{h}x{v}", "fwd_ms": f_ms, "bwd_ms": b_ms,
+                     "fwd_tflops": flop / f_ms / 1e9, "bwd_tflops": 3.0 * flop / b_ms / 1e9,
+                     "fwd_frac_of_fp32_peak": flop / f_ms / 1e9 / 157.3,
+                     "bwd_frac_of_fp32_peak": 3.0 * flop / b_ms / 1e9 / 157.3,
+                     "library_fp32_gemm_tflops": flop / g_ms / 1e9})
+        del hidden, weight
+    return {"what": "rlk_linear_logp_fwd / _bwd on fp32 inputs (v_mfma_f32_32x32x2_f32 tiles), "
+                    "TFLOP/s on 2NHV / 6NHV, peak 157.3 TFLOP/s", "rows": rows}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -647,6 +679,7 @@ def main() -> int:
                                                    "bitwise_repeatable", "roofline")}
         torch.cuda.empty_cache()
         extras["reference-published-shapes"] = bench_reference_shapes(torch)
+        extras["fp32-inputs"] = bench_fp32_inputs(torch)
         torch.cuda.empty_cache()
         result["extra_workloads"] = extras
 

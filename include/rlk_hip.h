@@ -69,10 +69,12 @@ const char* rlk_last_error(void);
  *            With strict_targets == 0 such a row yields logp = -lse (z_t = 0), which is what a
  *            vocab-parallel shard must return (csrc/cuda/fused_linear_logp_sm90.cu:256-280).
  *   dtype: RLK_DTYPE_BF16 / RLK_DTYPE_F16 with H % 8 == 0 and 16-byte aligned matrices run on the
- *   MFMA tiles; RLK_DTYPE_F32, other H or misaligned matrices run on scalar-FMA kernels (same
- *   math in fp32, H <= 12288) -- the counterpart of the reference's "unsupported dtype/shape falls
- *   back to the portable op" (rl_engine/kernels/ops/cuda/loss/linear_logp.py:45-55,350-351),
- *   except that here the portable op is HIP too.
+ *   16-bit MFMA tiles; RLK_DTYPE_F32, other H or misaligned matrices run on the fp32 matrix
+ *   instruction (operands widened to fp32 on the way into LDS, same tiling, any N, H, V >= 1) --
+ *   the counterpart of the reference's "unsupported dtype/shape falls back to the portable op"
+ *   (rl_engine/kernels/ops/cuda/loss/linear_logp.py:45-55,350-351), except that here the
+ *   portable op is a matrix-core HIP kernel too.  Every forward entry point below (static
+ *   scratch, two heads, folded GRPO epilogue) and the backward take both kinds of input.
  * ------------------------------------------------------------------------------------------ */
 int rlk_linear_logp_fwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                         size_t* bytes);

@@ -14,7 +14,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "librlk_hip.so")
 
 SOURCES = ["rlk_core.hip", "rlk_linear_logp.hip", "rlk_logp_scan.hip", "rlk_grpo.hip",
-           "rlk_generic.hip", "rlk_rmsnorm.hip"]
+           "rlk_wide.hip", "rlk_rmsnorm.hip"]
 
 # Packed-fp32 VALU forms are switched off for every device function of this library (the host pass
 # of hipcc warns that it does not know the feature; build() checks the device code instead).

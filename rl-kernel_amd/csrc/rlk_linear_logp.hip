@@ -12,11 +12,10 @@
 
 #include "rlk_gemm.hpp"
 #include "rlk_grpo.hpp"
+#include "rlk_tile_epilogue.hpp"
 
 namespace rlk {
 
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
 
 // ------------------------------------------------------------------------------------------- //
 // Forward
@@ -47,69 +46,6 @@ struct FwdArgs {
     int vtiles;      // vocab tiles of this launch
     float scale2;    // log2(e) / temperature
 };
-
-// Online-softmax update of one wavefront slab (kTM*32 vocab rows x kTN*32 tokens) held in `acc`.
-// GENERAL = false: no bias and no masked vocab rows (every tile full), the common case.
-// The target logit is picked up in the same pass that feeds the sum, so the captured value is
-// the very fp32 number that entered the softmax.
-template <bool GENERAL>
-__device__ inline void fwd_epilogue(const f32x16_t (&acc)[kTM][kTN], const FwdArgs& a,
-                                    const float* bias, int vw, int lane, const int (&tgt)[kTN],
-                                    float (&m)[kTN], float (&s)[kTN], float (&zt)[kTN])
-{
-    auto logit = [&](int i, int j, int r) -> float {
-        float z = acc[i][j][r];
-        if (GENERAL) {
-            const int v = vw + i * 32 + acc_row(r, lane);
-            if (bias != nullptr) z += bias[v < a.V ? v : a.V - 1];
-            if (v >= a.V) z = -INFINITY;
-        }
-        return z;
-    };
-#pragma unroll
-    for (int j = 0; j < kTN; ++j) {
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < kTM; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, logit(i, j, r));
-        __builtin_amdgcn_sched_barrier(0);
-        tmax *= a.scale2;
-        const float mnew = fmaxf(m[j], tmax);
-        const float mref = mnew == -INFINITY ? 0.f : mnew;
-        // register index (i*16 + r) of the target row in this lane, or -1
-        const int tl = tgt[j] - vw;
-        const int x = tl & 31;
-        const int etgt = (static_cast<unsigned>(tl) < static_cast<unsigned>(kTM * 32) && ((x >> 2) & 1) == (lane >> 5))
-                             ? ((tl >> 5) * 16 + (x >> 3) * 4 + (x & 3))
-                             : -1;
-        // four partial sums (fixed association) keep the exp results off a single add chain; the
-        // target capture runs only when some lane of the wavefront owns a target row in this slab
-        float ps[4] = {0.f, 0.f, 0.f, 0.f};
-        float zraw = 0.f;
-        if (__builtin_amdgcn_ballot_w64(etgt >= 0) != 0) {  // uniform
-#pragma unroll
-            for (int i = 0; i < kTM; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float z = logit(i, j, r);
-                    ps[r & 3] += __builtin_amdgcn_exp2f(fmaf(z, a.scale2, -mref));
-                    zraw = (etgt == i * 16 + r) ? z : zraw;
-                }
-        } else {
-#pragma unroll
-            for (int i = 0; i < kTM; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    ps[r & 3] += __builtin_amdgcn_exp2f(fmaf(logit(i, j, r), a.scale2, -mref));
-        }
-        const float sum = (ps[0] + ps[1]) + (ps[2] + ps[3]);
-        __builtin_amdgcn_sched_barrier(0);
-        s[j] = s[j] * __builtin_amdgcn_exp2f(m[j] - mref) + sum;
-        m[j] = mnew;
-        if (etgt >= 0) zt[j] = zraw * a.scale2;
-    }
-}
 
 // One workgroup = one block of 256 tokens x one contiguous range of vocab tiles.
 // GENERAL = false requires bias == null and covers only full vocab tiles [0, vtiles) split
@@ -379,33 +315,6 @@ struct DzArgs {
     int use_ignore;
     float scale2;
 };
-
-// Tiles of a launch are handed out round by round: workgroup b computes the tiles with linear ids
-// b, b + gridDim.x, b + 2 gridDim.x, ...  With a grid that is a multiple of 8, a workgroup keeps
-// its XCD from round to round, so every round forms the same L2-sharing patches as a launch with
-// one workgroup per tile would.
-struct TileWalk {
-    int lin, total, gm, gn;
-    __device__ inline TileWalk(int total_, int gm_, int gn_)
-        : lin(blockIdx.x), total(total_), gm(gm_), gn(gn_) {}
-    __device__ inline bool valid() const { return lin < total; }
-    __device__ inline bool has_next() const { return lin + static_cast<int>(gridDim.x) < total; }
-    __device__ inline void coords(bool next, int& tm, int& tn) const
-    {
-        xcd_tile(next ? lin + static_cast<int>(gridDim.x) : lin, total, gm, gn, 8, tm, tn);
-    }
-    __device__ inline void advance() { lin += static_cast<int>(gridDim.x); }
-};
-
-__device__ inline void zero_acc(f32x16_t (&acc)[kTM][kTN])
-{
-#pragma unroll
-    for (int i = 0; i < kTM; ++i)
-#pragma unroll
-        for (int j = 0; j < kTN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-}
 
 // LDS each wavefront needs to turn its part of a dZ tile into full rows: 64 tokens x 32 vocab
 // columns of 16-bit values, 64 bytes per token row, no padding.
@@ -1181,8 +1090,8 @@ int check_common(int64_t N, int32_t H, int64_t V, int dtype)
     return 0;
 }
 
-// The MFMA tiles take 16-bit inputs whose rows start on 16-byte boundaries; everything else runs
-// on the scalar-FMA kernels.
+// The 16-bit MFMA tiles take bf16 / f16 inputs whose rows start on 16-byte boundaries; everything
+// else runs on the fp32 matrix-core kernels (rlk_wide.hip).
 bool use_mfma(const void* hidden, const void* weight, int32_t H, int dtype)
 {
     return (dtype == RLK_DTYPE_BF16 || dtype == RLK_DTYPE_F16) && H % 8 == 0 &&
@@ -1580,16 +1489,6 @@ int rlk_linear_logp_fwd_grpo(const void* hidden, const void* weight, const float
     g.clip_hi = 1.f + clip_eps;
     g.beta = beta;
     g.blocks = grpo_blocks(N);
-    if (!use_mfma(hidden, weight, H, dtype)) {
-        // scalar-FMA forward, then the stand-alone epilogue (same values: it is the same math)
-        if (int rc = fwd_enqueue(hidden, weight, bias, targets, logp, lse, workspace, fwd, N, H, V,
-                                 vocab_start, dtype, temperature, ignore_index, use_ignore,
-                                 strict_targets, err_flag, stream))
-            return rc;
-        return rlk_grpo_loss_from_logp(logp, old_logp, ref_logp, advantages, adv_per_token, mask, N,
-                                       seq_len, clip_eps, beta, out3, ratio, kl_terms, d_cur, d_kl,
-                                       nullptr, g.partial, need - (fwd + 255) / 256 * 256, stream);
-    }
     return fwd_enqueue(hidden, weight, bias, targets, logp, lse, workspace, fwd, N, H, V, vocab_start,
                        dtype, temperature, ignore_index, use_ignore, strict_targets, err_flag, stream,
                        &g);
@@ -1615,16 +1514,6 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
         return rlk_fail(RLK_ERR_ARG, "strict_targets needs an err_flag to report through");
     const bool mfma = use_mfma(hidden, weight, H, dtype) &&
                       (second == nullptr || use_mfma(hidden, second->weight, H, dtype));
-    if (!mfma) {
-        if (epilogue != nullptr) return rlk_fail(RLK_ERR_UNSUPPORTED, "scalar path has no folded epilogue");
-        if (int rc = generic_fwd(hidden, weight, bias, targets, logp, lse, N, H, V, vocab_start, dtype,
-                                 temperature, ignore_index, use_ignore, strict_targets, err_flag, stream))
-            return rc;
-        if (second == nullptr) return 0;
-        return generic_fwd(hidden, second->weight, second->bias, targets, second->logp, second->lse, N,
-                           H, V, vocab_start, dtype, temperature, ignore_index, use_ignore, 0,
-                           err_flag, stream);
-    }
     size_t need = 0;
     rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &need);
     if (second != nullptr) need *= 2;
@@ -1648,8 +1537,10 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
     a.H = H;
     a.V = static_cast<int>(V);
     a.vocab_start = vocab_start;
-    // with two heads a bias on either sends both through the general launch
-    const FwdPlan plan = fwd_plan(N, V, bias != nullptr || (second != nullptr && second->bias != nullptr));
+    // with two heads a bias on either sends both through the general launch; the fp32 matrix-core
+    // kernels treat every tile as general
+    const FwdPlan plan =
+        fwd_plan(N, V, !mfma || bias != nullptr || (second != nullptr && second->bias != nullptr));
     a.row_blocks = plan.row_blocks;
     a.part_m = static_cast<float*>(workspace);
     a.part_s = a.part_m + static_cast<size_t>(plan.total_splits) * N;
@@ -1659,8 +1550,18 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
     a.part2_z = a.part2_s + static_cast<size_t>(plan.total_splits) * N;
     a.scale2 = kLog2e / temperature;
 
+    if (!mfma) {
+        if (int rc = wide_fwd_partials(hidden, weight, bias, targets, a.part_m, a.part_s, a.part_z,
+                                       plan.total_splits, N, H, V, vocab_start, dtype, temperature, stream))
+            return rc;
+        if (second != nullptr)
+            if (int rc = wide_fwd_partials(hidden, second->weight, second->bias, targets, a.part2_m,
+                                           a.part2_s, a.part2_z, plan.total_splits, N, H, V, vocab_start,
+                                           dtype, temperature, stream))
+                return rc;
+    }
     using G = TileGemm<Bf16, false, false, kBK>;  // same LDS footprint for f16
-    if (plan.n_fast > 0) {
+    if (mfma && plan.n_fast > 0) {
         a.n_split = plan.n_fast;
         a.split_lo = 0;
         a.tile_lo = 0;
@@ -1676,7 +1577,7 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
                                G::kSmemBytes, stream, a);
         }
     }
-    if (plan.n_gen > 0) {
+    if (mfma && plan.n_gen > 0) {
         a.n_split = plan.n_gen;
         a.split_lo = plan.n_fast;
         a.tile_lo = plan.fast_tiles;
@@ -1746,7 +1647,7 @@ int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t
     if (!bytes || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad workspace query");
     dz_budget_bytes = clamp_dz_budget(dz_budget_bytes);
     // large enough for either implementation (the choice also depends on pointer alignment)
-    const size_t a = bwd_plan(N, H, V, dz_budget_bytes).total, b = generic_bwd_workspace(N, H, V);
+    const size_t a = bwd_plan(N, H, V, dz_budget_bytes).total, b = wide_bwd_workspace(N, H, V, dz_budget_bytes);
     *bytes = a > b ? a : b;
     return 0;
 }
@@ -1800,13 +1701,10 @@ int rlk::linear_logp_bwd_accumulating(const float* grad_logp, const void* hidden
     if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
     if (reinterpret_cast<uintptr_t>(workspace) & 255)
         return rlk_fail(RLK_ERR_ARG, "workspace must be 256-byte aligned");
-    if (!use_mfma(hidden, weight, H, dtype)) {
-        if (accumulate && (d_weight || d_bias))
-            return rlk_fail(RLK_ERR_UNSUPPORTED, "the scalar path cannot add to existing gradients");
-        return generic_bwd(grad_logp, hidden, weight, bias, targets, lse, d_hidden, d_weight, d_bias,
-                           workspace, N, H, V, vocab_start, dtype, temperature, ignore_index,
-                           use_ignore, stream);
-    }
+    if (!use_mfma(hidden, weight, H, dtype))
+        return wide_bwd(grad_logp, hidden, weight, bias, targets, lse, d_hidden, d_weight, d_bias,
+                        workspace, dz_budget_bytes, N, H, V, vocab_start, dtype, temperature,
+                        ignore_index, use_ignore, accumulate, stream);
     const BwdPlan p = bwd_plan(N, H, V, dz_budget_bytes);
     int n_cu = 0;
     if (int rc = compute_units(&n_cu)) return rc;

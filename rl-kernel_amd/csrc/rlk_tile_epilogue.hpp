@@ -1,0 +1,103 @@
+// Pieces shared by the 16-bit MFMA kernels and the fp32 MFMA kernels of the fused linear-logprob
+// path: both work on the same 256 x 256 workgroup tile with the same wavefront grid and the same
+// accumulator layout, so the code that consumes a finished tile does not depend on the operand type.
+#pragma once
+#include "rlk_gemm.hpp"
+
+namespace rlk {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Online-softmax update of one wavefront slab (kTM*32 vocab rows x kTN*32 tokens) held in `acc`.
+// `a` supplies V (vocab rows of the shard) and scale2 (log2(e) / temperature).
+// GENERAL = false: no bias and no masked vocab rows (every tile full), the common case.
+// The target logit is picked up in the same pass that feeds the sum, so the captured value is
+// the very fp32 number that entered the softmax.
+template <bool GENERAL, class Args>
+__device__ inline void fwd_epilogue(const f32x16_t (&acc)[kTM][kTN], const Args& a,
+                                    const float* bias, int vw, int lane, const int (&tgt)[kTN],
+                                    float (&m)[kTN], float (&s)[kTN], float (&zt)[kTN])
+{
+    auto logit = [&](int i, int j, int r) -> float {
+        float z = acc[i][j][r];
+        if (GENERAL) {
+            const int v = vw + i * 32 + acc_row(r, lane);
+            if (bias != nullptr) z += bias[v < a.V ? v : a.V - 1];
+            if (v >= a.V) z = -INFINITY;
+        }
+        return z;
+    };
+#pragma unroll
+    for (int j = 0; j < kTN; ++j) {
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < kTM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, logit(i, j, r));
+        __builtin_amdgcn_sched_barrier(0);
+        tmax *= a.scale2;
+        const float mnew = fmaxf(m[j], tmax);
+        const float mref = mnew == -INFINITY ? 0.f : mnew;
+        // register index (i*16 + r) of the target row in this lane, or -1
+        const int tl = tgt[j] - vw;
+        const int x = tl & 31;
+        const int etgt = (static_cast<unsigned>(tl) < static_cast<unsigned>(kTM * 32) && ((x >> 2) & 1) == (lane >> 5))
+                             ? ((tl >> 5) * 16 + (x >> 3) * 4 + (x & 3))
+                             : -1;
+        // four partial sums (fixed association) keep the exp results off a single add chain; the
+        // target capture runs only when some lane of the wavefront owns a target row in this slab
+        float ps[4] = {0.f, 0.f, 0.f, 0.f};
+        float zraw = 0.f;
+        if (__builtin_amdgcn_ballot_w64(etgt >= 0) != 0) {  // uniform
+#pragma unroll
+            for (int i = 0; i < kTM; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float z = logit(i, j, r);
+                    ps[r & 3] += __builtin_amdgcn_exp2f(fmaf(z, a.scale2, -mref));
+                    zraw = (etgt == i * 16 + r) ? z : zraw;
+                }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kTM; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    ps[r & 3] += __builtin_amdgcn_exp2f(fmaf(logit(i, j, r), a.scale2, -mref));
+        }
+        const float sum = (ps[0] + ps[1]) + (ps[2] + ps[3]);
+        __builtin_amdgcn_sched_barrier(0);
+        s[j] = s[j] * __builtin_amdgcn_exp2f(m[j] - mref) + sum;
+        m[j] = mnew;
+        if (etgt >= 0) zt[j] = zraw * a.scale2;
+    }
+}
+
+// Tiles of a launch are handed out round by round: workgroup b computes the tiles with linear ids
+// b, b + gridDim.x, b + 2 gridDim.x, ...  With a grid that is a multiple of 8, a workgroup keeps
+// its XCD from round to round, so every round forms the same L2-sharing patches as a launch with
+// one workgroup per tile would.
+struct TileWalk {
+    int lin, total, gm, gn;
+    __device__ inline TileWalk(int total_, int gm_, int gn_)
+        : lin(blockIdx.x), total(total_), gm(gm_), gn(gn_) {}
+    __device__ inline bool valid() const { return lin < total; }
+    __device__ inline bool has_next() const { return lin + static_cast<int>(gridDim.x) < total; }
+    __device__ inline void coords(bool next, int& tm, int& tn) const
+    {
+        xcd_tile(next ? lin + static_cast<int>(gridDim.x) : lin, total, gm, gn, 8, tm, tn);
+    }
+    __device__ inline void advance() { lin += static_cast<int>(gridDim.x); }
+};
+
+__device__ inline void zero_acc(f32x16_t (&acc)[kTM][kTN])
+{
+#pragma unroll
+    for (int i = 0; i < kTM; ++i)
+#pragma unroll
+        for (int j = 0; j < kTN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+}
+
+}  // namespace rlk

@@ -145,10 +145,9 @@ class RocmFusedGRPOStepOp:
         if lm_head_weight.size(-1) != hidden.size(-1):
             raise ValueError(f"hidden dim {hidden.size(-1)} must match lm_head_weight dim "
                              f"{lm_head_weight.size(-1)}")
-        if not LL.hip_path_supported(hidden, lm_head_weight) or hidden.dtype == torch.float32 \
-                or hidden.size(-1) % 8 != 0:
-            raise NotImplementedError("RocmFusedGRPOStepOp needs bf16 / f16 hidden and weight of one "
-                                      "dtype on one GPU with a hidden size that is a multiple of 8")
+        if not LL.hip_path_supported(hidden, lm_head_weight):
+            raise NotImplementedError("RocmFusedGRPOStepOp needs hidden and weight of one dtype "
+                                      "(bf16, f16 or f32) on one GPU")
         ids = token_ids.to(device=hidden.device).long()
         mask = None
         if completion_mask is not None:

@@ -47,7 +47,7 @@ def _out_of_range_error(target_1d: torch.Tensor, vocab: int, ignore_index: Optio
 
 def hip_path_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     """bf16 / f16 / f32 tensors of one dtype on one GPU.  bf16/f16 with a hidden size that is a
-    multiple of 8 run on the MFMA tiles, the rest on the scalar-FMA kernels (H <= 12288)."""
+    multiple of 8 run on the 16-bit MFMA tiles, the rest on the fp32 matrix-core kernels."""
     return (
         hidden.is_cuda
         and weight.is_cuda
@@ -57,25 +57,35 @@ def hip_path_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     )
 
 
-_scalar_path_warned = False
+def _common_dtype(hidden: torch.Tensor, weight: torch.Tensor):
+    """Hidden states and weight of different supported dtypes (an fp32 head over bf16 activations,
+    say) are both widened to fp32, which is exact, and run on the fp32 kernels; autograd casts the
+    gradients back.  The reference's portable ops upcast the same way
+    (rl_engine/kernels/ops/pytorch/loss/linear_logp.py:17-22)."""
+    if hidden.dtype != weight.dtype and hidden.dtype in _DTYPES and weight.dtype in _DTYPES:
+        return hidden.float(), weight.float()
+    return hidden, weight
 
 
-def _warn_if_scalar_path(hidden_2d: torch.Tensor, weight: torch.Tensor) -> None:
-    """The MFMA tiles take bf16/f16 with H % 8 == 0 and 16-byte aligned matrices; everything else
-    runs on scalar-FMA kernels that are meant for small correctness-sized problems.  Say so once
-    when a large problem ends up there."""
-    global _scalar_path_warned
-    if _scalar_path_warned:
+_wide_path_warned = False
+
+
+def _warn_if_wide_path(hidden_2d: torch.Tensor, weight: torch.Tensor) -> None:
+    """The 16-bit MFMA tiles take bf16/f16 with H % 8 == 0 and 16-byte aligned matrices; 16-bit
+    inputs that miss that run on the fp32 matrix instruction at roughly a tenth of the rate.  Say so
+    once when a large problem ends up there."""
+    global _wide_path_warned
+    if _wide_path_warned or hidden_2d.dtype == torch.float32:
         return
     n, h = hidden_2d.shape
-    on_mfma = (hidden_2d.dtype in (torch.bfloat16, torch.float16) and h % 8 == 0
-               and hidden_2d.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+    on_mfma = (h % 8 == 0 and hidden_2d.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
     if not on_mfma and n * h * weight.size(0) > (1 << 33):
-        _scalar_path_warned = True
+        _wide_path_warned = True
         logger.warning(
-            "linear_logp: %s inputs with H=%d run on the scalar-FMA kernels (the MFMA path takes "
-            "bf16/f16, H %% 8 == 0, 16-byte aligned matrices); expect this %d x %d x %d problem "
-            "to be slow", str(hidden_2d.dtype), h, n, h, weight.size(0))
+            "linear_logp: %s inputs with H=%d run on the fp32 matrix-core kernels (the 16-bit MFMA "
+            "path takes H %% 8 == 0 and 16-byte aligned matrices); expect this %d x %d x %d problem "
+            "to run at about a tenth of the 16-bit rate", str(hidden_2d.dtype), h, n, h,
+            weight.size(0))
 
 
 def fused_linear_logp_forward(
@@ -104,7 +114,7 @@ def fused_linear_logp_forward(
     err = torch.zeros(1, device=dev, dtype=torch.int32)
     if n == 0:  # nothing to launch
         return logp, lse, err
-    _warn_if_scalar_path(hidden_2d, weight)
+    _warn_if_wide_path(hidden_2d, weight)
     need = _native.ctypes.c_size_t(0)
     dt = _DTYPES[hidden_2d.dtype]
     _native.check(lib.rlk_linear_logp_fwd_workspace_bytes(n, h, v, dt, _native.ctypes.byref(need)),
@@ -146,7 +156,7 @@ def fused_linear_logp_forward_pair(
     err = torch.zeros(1, device=dev, dtype=torch.int32)
     if n == 0:
         return (*outs, err)
-    _warn_if_scalar_path(hidden_2d, weight)
+    _warn_if_wide_path(hidden_2d, weight)
     need = _native.ctypes.c_size_t(0)
     dt = _DTYPES[hidden_2d.dtype]
     _native.check(lib.rlk_linear_logp_fwd_pair_workspace_bytes(n, h, v, dt, _native.ctypes.byref(need)),
@@ -187,7 +197,7 @@ def fused_norm_linear_logp_forward(
     err = torch.zeros(1, device=dev, dtype=torch.int32)
     if n == 0:
         return logp, lse, err
-    _warn_if_scalar_path(x_2d, weight)
+    _warn_if_wide_path(x_2d, weight)
     need = _native.ctypes.c_size_t(0)
     dt = _DTYPES[x_2d.dtype]
     _native.check(lib.rlk_linear_logp_rmsnorm_fwd_workspace_bytes(n, h, v, dt, _native.ctypes.byref(need)),
@@ -492,10 +502,12 @@ class RocmFusedLinearLogpOp:
         if global_vocab_size is not None and int(global_vocab_size) != vocab:
             raise ValueError("global_vocab_size differs from the local vocab size, but no "
                              "multi-rank tensor-parallel group was provided.")
+        if norm_weight is None:
+            hidden, lm_head_weight = _common_dtype(hidden, lm_head_weight)
         if not hip_path_supported(hidden, lm_head_weight):
             raise NotImplementedError(
-                "RocmFusedLinearLogpOp needs hidden and lm_head_weight of one dtype "
-                "(bf16, f16 or f32) on the same GPU")
+                "RocmFusedLinearLogpOp needs hidden and lm_head_weight in bf16, f16 or f32 on the "
+                "same GPU (and of one dtype when norm_weight is given)")
         if norm_weight is not None:
             if norm_weight.dim() != 1 or norm_weight.shape[0] != hidden.size(-1):
                 raise ValueError(f"norm_weight must be 1-D of size hidden.shape[-1]={hidden.size(-1)}, "

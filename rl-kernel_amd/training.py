@@ -78,17 +78,17 @@ def grpo_loss_step(hidden: torch.Tensor, lm_head: torch.nn.Linear, token_ids: to
                    registry=None, fuse_epilogue: bool = True) -> GRPOStepResult:
     """hidden -> fused logp -> group-normalised advantages -> fused GRPO loss (call
     ``result.loss.backward()`` for dH / dW / db).  Ops come from the kernel registry.  With
-    ``fuse_epilogue`` (16-bit hidden states, hidden size a multiple of 8) the loss terms leave the
+    ``fuse_epilogue`` (hidden states and head of one dtype on the GPU) the loss terms leave the
     forward's last launch (``grpo_step_from_hidden``); the values are the same bits either way."""
     if registry is None:
         from .registry import kernel_registry as registry
     linear_logp = registry.get_op("linear_logp")
     loss_op = registry.get_op("grpo_loss_from_logp")
-    fusable = (fuse_epilogue and hidden.dim() >= 2 and hidden.size(-1) % 8 == 0
-               and hidden.dtype in (torch.bfloat16, torch.float16))
+    if not isinstance(lm_head, torch.nn.Linear):
+        raise TypeError("model must expose an lm_head torch.nn.Linear for linear_logp")
+    fusable = (fuse_epilogue and hidden.dim() >= 2 and lm_head.weight.dtype == hidden.dtype
+               and hidden.dtype in (torch.bfloat16, torch.float16, torch.float32))
     if fusable:
-        if not isinstance(lm_head, torch.nn.Linear):
-            raise TypeError("model must expose an lm_head torch.nn.Linear for linear_logp")
         step_op = registry.get_op("grpo_step_from_hidden")
         adv = loss_op.group_advantages(rewards, samples_per_prompt=samples_per_prompt,
                                        group_boundaries=group_boundaries)

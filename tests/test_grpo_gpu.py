@@ -230,6 +230,8 @@ def test_fused_step_linear_logp_into_grpo_epilogue(dev, ops):
     (4, 300, 128, 2304, torch.float16, True, True),       # several loss blocks' worth of threads
     (3, 50, 64, 1000, torch.bfloat16, False, False),      # no reference model: KL term off
     (64, 512, 256, 4096, torch.bfloat16, False, True),    # 32768 tokens: 8 loss blocks, vocab splits
+    (5, 60, 50, 600, torch.float32, True, True),          # fp32 inputs: behind the fp32 matrix-core kernels
+    (6, 33, 36, 300, torch.bfloat16, False, True),        # 16-bit with H % 8 != 0: same
 ])
 def test_epilogue_folded_into_the_forward_equals_the_two_step_route(dev, ops, b, t, h, v, dtype,
                                                                     per_token_adv, with_ref):
