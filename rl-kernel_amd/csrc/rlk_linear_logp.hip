@@ -48,8 +48,9 @@ struct FwdArgs {
 };
 
 // One workgroup = one block of 256 tokens x one contiguous range of vocab tiles.
-// GENERAL = false requires bias == null and covers only full vocab tiles [0, vtiles) split
-// n_split ways; GENERAL = true handles bias and/or masked rows over tiles [tile_lo, tile_lo+vtiles).
+// GENERAL = false covers only full vocab tiles [0, vtiles) split n_split ways (a bias is added to
+// the finished tile before the softmax update); GENERAL = true handles masked rows over tiles
+// [tile_lo, tile_lo+vtiles).
 template <class T, int BK, bool GENERAL>
 __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
 {
@@ -162,6 +163,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
                                                : (head + 1 < n_heads ? tile_origin(head + 1, t0)
                                                                      : tile_origin(head, vt));
                 Dtl::tile(st, next, B.base, acc, smem);
+                const float* bias = head == 0 ? a.bias : a.bias2;
+                if (bias != nullptr) add_bias(acc, bias, vt * 256 + wm * (TM * 32), lane);  // uniform
                 fwd_epilogue<GENERAL>(acc, a, nullptr, vt * 256 + wm * (TM * 32), lane, tgt, m, s, zt);
             }
             if (head == 0)
@@ -185,6 +188,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
                 Gemm::run(A, B, a.H, acc, smem);
+                if (!GENERAL && bias != nullptr) add_bias(acc, bias, v0 + wm * (TM * 32), lane);  // uniform
                 fwd_epilogue<GENERAL>(acc, a, bias, v0 + wm * (TM * 32), lane, tgt, m, s, zt);
             }
             if (head == 0)
@@ -417,7 +421,7 @@ __device__ inline void dz_epilogue(const f32x16_t (&acc)[kTM][kTN], const DzArgs
     });
 }
 
-// GENERAL = false: no bias, every vocab tile of the launch is full.
+// GENERAL = false: every vocab tile of the launch is full (a bias is added to the finished tile).
 // CHAIN (needs !GENERAL, full token tiles, H a multiple of BK and >= 2 BK): the workgroup walks
 // its tiles through one pipeline; while a tile's epilogue runs, the first K steps of the next
 // tile are already on their way into LDS.
@@ -447,6 +451,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
             zero_acc(acc);
             Dtl::template tile<true, kDzStores / 2>(st, w_origin(nvt), h_origin(ntt), acc, smem, true);
             if (more) Dtl::fetch_ahead(st, smem);
+            if (a.bias != nullptr)  // uniform
+                add_bias(acc, a.bias, (vt + a.v_tile_lo) * 256 + (wave / kWN) * (kTM * 32), threadIdx.x & 63);
             dz_epilogue<T, GENERAL>(acc, a, vt + a.v_tile_lo, tt, stage);
             if (!more) break;
             walk.advance();
@@ -462,6 +468,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
             Operand B{h_origin(tt), a.H, min(256, a.tok_valid - tok0)};
             zero_acc(acc);
             Gemm::run(A, B, a.H, acc, smem);  // ends with a barrier: LDS is free
+            if (!GENERAL && a.bias != nullptr)  // uniform
+                add_bias(acc, a.bias, v0 + (wave / kWN) * (kTM * 32), threadIdx.x & 63);
             dz_epilogue<T, GENERAL>(acc, a, vt + a.v_tile_lo, tt, smem + wave * kDzStageBytes);
             if (!walk.has_next()) break;
             walk.advance();
@@ -805,17 +813,45 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
     }
 }
 
-// db[v] (+)= sum_tok dZ[tok][v], tokens in ascending order (fixed order).
-__global__ void linear_logp_db_kernel(const uint16_t* dz, int64_t ldz, int tok_valid, int v_valid,
-                                      const float* scales, float* db, int accumulate, int dtype)
+// db[v] (+)= sum_tok dZ[tok][v] in two fixed-order levels.  Level 1: one workgroup per (256
+// columns) x (256-token tile); a thread owns 8 columns (one 16-byte load per row) of every eighth
+// row, the eight row groups are added in order through LDS: part[tile][v].  The dZ block is written
+// in whole tiles (padding rows and columns hold zeros), so no row or column check is needed here.
+template <class T>
+__global__ __launch_bounds__(256) void linear_logp_db_partial_kernel(const uint16_t* dz, int64_t ldz, float* part,
+                                                                     int64_t part_ld)
+{
+    __shared__ float red[8][256];
+    const int cg = threadIdx.x & 31, rg = threadIdx.x >> 5;
+    const int v0 = blockIdx.x * 256 + cg * 8;
+    const uint16_t* p = dz + (static_cast<int64_t>(blockIdx.y) * 256 + rg) * ldz + v0;
+    float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int k = 0; k < 32; ++k) {
+        const u32x4_t w = *reinterpret_cast<const u32x4_t*>(p + static_cast<int64_t>(k) * 8 * ldz);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            sum[2 * e] += T::to_float(static_cast<uint16_t>(w[e] & 0xffffu));
+            sum[2 * e + 1] += T::to_float(static_cast<uint16_t>(w[e] >> 16));
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red[rg][cg * 8 + e] = sum[e];
+    __syncthreads();
+    float acc = red[0][threadIdx.x];
+#pragma unroll
+    for (int r = 1; r < 8; ++r) acc += red[r][threadIdx.x];
+    part[static_cast<int64_t>(blockIdx.y) * part_ld + blockIdx.x * 256 + threadIdx.x] = acc;
+}
+
+// Level 2: the token tiles of the block in ascending order, times 1 / loss_scale.
+__global__ void linear_logp_db_finish_kernel(const float* part, int64_t part_ld, int tok_tiles, int v_valid,
+                                             const float* scales, float* db, int accumulate)
 {
     const int v = blockIdx.x * blockDim.x + threadIdx.x;
     if (v >= v_valid) return;
-    float sum = 0.f;
-    for (int t = 0; t < tok_valid; ++t) {
-        const uint16_t x = dz[static_cast<int64_t>(t) * ldz + v];
-        sum += dtype == 0 ? Bf16::to_float(x) : F16::to_float(x);
-    }
+    float sum = part[v];
+    for (int t = 1; t < tok_tiles; ++t) sum += part[static_cast<int64_t>(t) * part_ld + v];
     sum *= scales[1];
     db[v] = accumulate ? db[v] + sum : sum;
 }
@@ -929,13 +965,13 @@ int split_count(int row_blocks, int tiles)
     return s;
 }
 
-FwdPlan fwd_plan(int64_t N, int64_t V, bool has_bias)
+FwdPlan fwd_plan(int64_t N, int64_t V, bool all_general)
 {
     FwdPlan p;
     p.row_blocks = static_cast<int>((N + 255) / 256);
     const int all = static_cast<int>((V + 255) / 256);
     const int full = static_cast<int>(V / 256);
-    p.fast_tiles = has_bias ? 0 : full;
+    p.fast_tiles = all_general ? 0 : full;
     p.gen_tiles = all - p.fast_tiles;
     p.n_fast = split_count(p.row_blocks, p.fast_tiles);
     p.n_gen = split_count(p.row_blocks, p.gen_tiles);
@@ -966,7 +1002,8 @@ struct BwdPlan {
     size_t dz_bytes;
     size_t acc_bytes;
     size_t part_bytes;
-    size_t scales_off, dz_off, acc_off, part_off, total;
+    size_t db_bytes;
+    size_t scales_off, dz_off, acc_off, part_off, db_off, total;
 };
 
 // Cost of the three launches of one dZ block of ct x pt tiles, in K steps of one CU: a launch of
@@ -1060,7 +1097,10 @@ BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
     }
     p.part_bytes = p.ksplit > 1 ? static_cast<size_t>(p.ksplit) * p.tok_chunk * H * 4 : 0;
     p.part_off = p.acc_off + align_up(p.acc_bytes, 256);
-    p.total = p.part_off + align_up(p.part_bytes, 256);
+    // per-token-tile column sums of the dZ block (d_bias): 1 KiB per dZ tile
+    p.db_bytes = static_cast<size_t>(best_ct) * p.v_piece * 4;
+    p.db_off = p.part_off + align_up(p.part_bytes, 256);
+    p.total = p.db_off + align_up(p.db_bytes, 256);
     memo = Key{N, V, H, budget, p};
     return p;
 }
@@ -1249,9 +1289,8 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             d.accumulate = ci > 0 || c.accumulate != 0;
 
             // dZ block: full vocab tiles through the fast variant (chained through one pipeline
-            // when the token tiles are full too), the rest (all of them when there is a bias)
-            // through the general one
-            const int fast_tiles = c.bias ? 0 : v_valid / 256;
+            // when the token tiles are full too), the ragged last one through the general one
+            const int fast_tiles = v_valid / 256;
             const int gen_tiles = v_tiles - fast_tiles;
             const bool k_ok = H % kBK == 0 && H >= 2 * kBK;
             if (fast_tiles > 0) {
@@ -1302,9 +1341,12 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
                                        dim3(kThreads), GW::kSmemBytes, stream, d);
             }
             if (c.d_bias != nullptr) {
-                hipLaunchKernelGGL(linear_logp_db_kernel, dim3((v_valid + 255) / 256), dim3(256), 0,
-                                   stream, dz, p.ldz, tok_valid, v_valid, scales, c.d_bias + v_lo,
-                                   (ci > 0 || c.accumulate != 0) ? 1 : 0, c.dtype);
+                float* db_part = reinterpret_cast<float*>(ws + p.db_off);
+                hipLaunchKernelGGL(linear_logp_db_partial_kernel<T>, dim3(v_tiles, tok_tiles), dim3(256), 0,
+                                   stream, dz, p.ldz, db_part, static_cast<int64_t>(p.v_piece));
+                hipLaunchKernelGGL(linear_logp_db_finish_kernel, dim3((v_valid + 255) / 256), dim3(256), 0,
+                                   stream, db_part, static_cast<int64_t>(p.v_piece), tok_tiles, v_valid,
+                                   scales, c.d_bias + v_lo, (ci > 0 || c.accumulate != 0) ? 1 : 0);
             }
             if (int rc = check_launch("linear_logp backward launch failed")) return rc;
         }
@@ -1537,10 +1579,8 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
     a.H = H;
     a.V = static_cast<int>(V);
     a.vocab_start = vocab_start;
-    // with two heads a bias on either sends both through the general launch; the fp32 matrix-core
-    // kernels treat every tile as general
-    const FwdPlan plan =
-        fwd_plan(N, V, !mfma || bias != nullptr || (second != nullptr && second->bias != nullptr));
+    // the fp32 matrix-core kernels treat every tile as general
+    const FwdPlan plan = fwd_plan(N, V, !mfma);
     a.row_blocks = plan.row_blocks;
     a.part_m = static_cast<float*>(workspace);
     a.part_s = a.part_m + static_cast<size_t>(plan.total_splits) * N;

@@ -73,6 +73,27 @@ __device__ inline void fwd_epilogue(const f32x16_t (&acc)[kTM][kTN], const Args&
     }
 }
 
+// acc += bias of a full tile: `vw` is the first vocab row of this wavefront's slab, relative to
+// bias[0].  A lane holds quads of four consecutive vocab rows, so the bias arrives in 16-byte
+// loads that are the same for every lane of a half-wave (one broadcast request each).
+__device__ inline void add_bias(f32x16_t (&acc)[kTM][kTN], const float* bias, int vw, int lane)
+{
+#pragma unroll
+    for (int i = 0; i < kTM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float* p = bias + vw + i * 32 + 8 * q + 4 * (lane >> 5);
+            const float b0 = p[0], b1 = p[1], b2 = p[2], b3 = p[3];
+#pragma unroll
+            for (int j = 0; j < kTN; ++j) {
+                acc[i][j][q * 4 + 0] += b0;
+                acc[i][j][q * 4 + 1] += b1;
+                acc[i][j][q * 4 + 2] += b2;
+                acc[i][j][q * 4 + 3] += b3;
+            }
+        }
+}
+
 // Tiles of a launch are handed out round by round: workgroup b computes the tiles with linear ids
 // b, b + gridDim.x, b + 2 gridDim.x, ...  With a grid that is a multiple of 8, a workgroup keeps
 // its XCD from round to round, so every round forms the same L2-sharing patches as a launch with

@@ -60,6 +60,9 @@ CASES = [
     ((300,), 64, 40000, torch.bfloat16, False, 1.0, 0.0),    # one K step, several tiles per workgroup
     ((300,), 128, 40000, torch.float16, False, 0.7, 0.1),    # two K steps, several tiles per workgroup
     ((700,), 192, 70000, torch.bfloat16, False, 1.0, 0.0),
+    ((512,), 256, 2304, torch.bfloat16, True, 0.7, 0.05),    # bias on full tiles: streamed forward, chained dZ
+    ((1024,), 128, 5000, torch.float16, True, 1.0, 0.0),     # bias, full tiles + ragged last tile
+    ((300,), 64, 40000, torch.bfloat16, True, 1.3, 0.1),     # bias, ragged token tile (unchained dZ)
 ]
 
 

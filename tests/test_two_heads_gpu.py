@@ -20,8 +20,9 @@ def dev():
     (300, 64, 1000, torch.bfloat16, False, 1.0),       # ragged token block and vocab tile
     (1500, 256, 9000, torch.bfloat16, False, 0.7),     # several vocab splits + a general tail tile
     (700, 128, 2304, torch.float16, False, 1.0),       # full tiles only: both heads in one pipeline
-    (257, 64, 513, torch.float16, True, 1.3),          # biased heads: general path for both
-    (64, 20, 300, torch.float32, True, 1.0),           # fp32: scalar path
+    (257, 64, 513, torch.float16, True, 1.3),          # biased heads, ragged tiles
+    (600, 128, 2304, torch.bfloat16, True, 0.7),       # biased heads on full tiles: each head adds its own bias
+    (64, 20, 300, torch.float32, True, 1.0),           # fp32 matrix-core kernels
     (4096, 1024, 40960, torch.bfloat16, False, 1.0),   # many tiles per workgroup and head
 ])
 def test_pair_forward_equals_two_single_forwards(dev, n, h, v, dtype, bias, temp):
