@@ -188,9 +188,14 @@ struct WideIO {
 };
 
 // Workgroup tile contraction on the fp32 matrix instruction: acc[i][j] += A rows x B rows over
-// k in [0, K).  Two LDS stages; the global loads of K step kt+1 are in flight while step kt is
-// multiplied (one MFMA of 32 x 32 x 2 takes 16 passes, so a stage is 64 MFMAs = 4096 cycles per
-// wavefront against a dozen fragment reads and 4 global loads: the loop is bound by the matrix pipe).
+// k in [0, K).  Two LDS stages and one barrier per stage, placed in the middle of the stage's
+// MFMAs so that every memory latency has matrix work in front of it:
+//   stage kt:  LDS stores of stage kt+1 (fetched one stage ago), global loads of stage kt+2,
+//              fragment reads of the second half, 32 MFMAs of the first half,
+//              barrier (stage kt+1 is now complete, nobody reads stage kt from LDS any more),
+//              fragment reads of the first half of stage kt+1, 32 MFMAs of the second half.
+// One MFMA of 32 x 32 x 2 takes 16 passes, so a stage is 4096 matrix cycles per wavefront against a
+// dozen fragment reads and 4 global loads: the loop is bound by the matrix pipe.
 // All 512 threads must call it (it barriers); on return LDS may be reused.
 template <int DTA, int DTB, bool A_KMAJOR, bool B_KMAJOR>
 struct WideGemm {
@@ -198,6 +203,27 @@ struct WideGemm {
     using IOB = WideIO<DTB, B_KMAJOR>;
     static constexpr int kStageFloats = IOA::kFloats + IOB::kFloats;
     static constexpr int kSmemBytes = 2 * kStageFloats * 4;
+
+    __device__ static inline void frags(const float* stage, int wm, int wn, int half, f32x4_t (&fa)[kTM],
+                                        f32x4_t (&fb)[kTN])
+    {
+#pragma unroll
+        for (int i = 0; i < kTM; ++i) fa[i] = IOA::frag(stage, wm * (kTM * 32) + i * 32, half);
+#pragma unroll
+        for (int j = 0; j < kTN; ++j) fb[j] = IOB::frag(stage + IOA::kFloats, wn * (kTN * 32) + j * 32, half);
+    }
+
+    __device__ static inline void multiply(const f32x4_t (&fa)[kTM], const f32x4_t (&fb)[kTN],
+                                           f32x16_t (&acc)[kTM][kTN])
+    {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+            for (int i = 0; i < kTM; ++i)
+#pragma unroll
+                for (int j = 0; j < kTN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][kk], fb[j][kk], acc[i][j], 0, 0, 0);
+    }
 
     __device__ static inline void run(const WideOperand& A, const WideOperand& B, int K,
                                       f32x16_t (&acc)[kTM][kTN], char* smem_c)
@@ -221,7 +247,16 @@ struct WideGemm {
             IOA::store(smem, ra[g], g);
             IOB::store(smem + IOA::kFloats, rb[g], g);
         }
+        if (nk > 1) {  // uniform
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                ra[g] = la.load(1, g);
+                rb[g] = lb.load(1, g);
+            }
+        }
         __syncthreads();
+        f32x4_t fa0[kTM], fb0[kTN], fa1[kTM], fb1[kTN];
+        frags(smem, wm, wn, 0, fa0, fb0);
         for (int kt = 0; kt < nk; ++kt) {
             const float* cur = smem + (kt & 1) * kStageFloats;
             float* nxt = smem + ((kt + 1) & 1) * kStageFloats;
@@ -229,34 +264,24 @@ struct WideGemm {
             if (more) {
 #pragma unroll
                 for (int g = 0; g < 2; ++g) {
-                    ra[g] = la.load(kt + 1, g);
-                    rb[g] = lb.load(kt + 1, g);
-                }
-            }
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                f32x4_t fa[kTM], fb[kTN];
-#pragma unroll
-                for (int i = 0; i < kTM; ++i) fa[i] = IOA::frag(cur, wm * (kTM * 32) + i * 32, half);
-#pragma unroll
-                for (int j = 0; j < kTN; ++j) fb[j] = IOB::frag(cur + IOA::kFloats, wn * (kTN * 32) + j * 32, half);
-#pragma unroll
-                for (int kk = 0; kk < 4; ++kk)
-#pragma unroll
-                    for (int i = 0; i < kTM; ++i)
-#pragma unroll
-                        for (int j = 0; j < kTN; ++j)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][kk], fb[j][kk], acc[i][j], 0, 0, 0);
-            }
-            if (more) {
-#pragma unroll
-                for (int g = 0; g < 2; ++g) {
                     IOA::store(nxt, ra[g], g);
                     IOB::store(nxt + IOA::kFloats, rb[g], g);
                 }
             }
+            if (kt + 2 < nk) {
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    ra[g] = la.load(kt + 2, g);
+                    rb[g] = lb.load(kt + 2, g);
+                }
+            }
+            frags(cur, wm, wn, 1, fa1, fb1);
+            multiply(fa0, fb0, acc);
             __syncthreads();
+            if (more) frags(nxt, wm, wn, 0, fa0, fb0);
+            multiply(fa1, fb1, acc);
         }
+        __syncthreads();
     }
 };
 

@@ -59,7 +59,8 @@ def test_backward_workspace_is_bounded_in_token_count(native):
         assert lib.rlk_linear_logp_bwd_workspace_bytes(n, 4096, 128256, 0, 0, ctypes.byref(need)) == 0
         sizes.append(need.value)
     # scratch does not grow with G = 64 ... 2048: one dZ block (<= 256 MiB) + fp32 dH chunk
-    assert max(sizes) <= (384 << 20) + 4096, sizes
+    # (<= 128 MiB) + the d_bias column sums per token tile (1 KiB per dZ tile, <= 2 MiB)
+    assert max(sizes) <= (386 << 20) + 4096, sizes
     assert max(sizes) <= 1 << 30                # <= 1 GiB extra HBM
     assert sizes[0] == sizes[1] == sizes[2]     # identical for G = 64, 128, 256
     need = ctypes.c_size_t(0)
@@ -157,7 +158,8 @@ def test_backward_plan_keeps_in_tile_offsets_within_32_bits(native, n, h, v, bud
     assert tok_chunk * n_chunks >= n and v_piece * n_pieces >= v
     need = ctypes.c_size_t(0)
     assert lib.rlk_linear_logp_bwd_workspace_bytes(n, h, v, 0, budget, ctypes.byref(need)) == 0
-    assert need.value <= (3 << 30) + (1 << 20)          # block + fp32 dH chunk <= 1.5 x 2 GiB
+    # block + fp32 dH chunk <= 1.5 x 2 GiB, + the d_bias column sums (1 KiB per 128 KiB dZ tile)
+    assert need.value <= (3 << 30) + (33 << 20)
 
 
 def test_compiled_pytorch_binding_exports_the_reference_symbol_names(native):
