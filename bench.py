@@ -72,6 +72,9 @@ WORKLOADS = {
                         ignore_frac=0.0, scan=True),
     "small": dict(tokens=4096, hidden=1024, vocab=32768, dtype="bf16", temperature=1.0,
                   ignore_frac=0.0),
+    # fp32 hidden states and head on the fp32 matrix instruction (two shapes, see bench_fp32_inputs)
+    "fp32-inputs": dict(tokens=4096, hidden=2048, vocab=32768, dtype="f32", temperature=1.0,
+                        ignore_frac=0.0, fp32=True),
 }
 
 # linear_logp latencies the reference publishes (docs/operators/linear-logp.md:116-132 of the
@@ -632,6 +635,18 @@ def main() -> int:
     if cfg.get("scan"):
         result = bench_scan(torch, args.steps, args.warmup, cfg)
         result["device"] = device_info(torch)
+        print(json.dumps(result))
+        return 0
+
+    if cfg.get("fp32"):
+        r = bench_fp32_inputs(torch)
+        row = r["rows"][0]
+        result = dict(common)
+        result.update({"metric": "linear_logp tokens/s (fwd+bwd)", "unit": "tokens/s", "dtype": "f32",
+                       "value": 4096 / ((row["fwd_ms"] + row["bwd_ms"]) * 1e-3),
+                       "ms_per_step": row["fwd_ms"] + row["bwd_ms"],
+                       "config": {"workload": "fp32-inputs: " + row["shape"] + " fp32, fwd + bwd"},
+                       "fp32": r, "device": device_info(torch)})
         print(json.dumps(result))
         return 0
 

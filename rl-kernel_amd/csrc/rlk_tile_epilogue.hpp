@@ -98,6 +98,9 @@ __device__ inline void add_bias(f32x16_t (&acc)[kTM][kTN], const float* bias, in
 // b, b + gridDim.x, b + 2 gridDim.x, ...  With a grid that is a multiple of 8, a workgroup keeps
 // its XCD from round to round, so every round forms the same L2-sharing patches as a launch with
 // one workgroup per tile would.
+#ifndef RLK_WALK_PATCH
+#define RLK_WALK_PATCH 8  // tile rows of the patch the 32 workgroups of one XCD cover per round
+#endif
 struct TileWalk {
     int lin, total, gm, gn;
     __device__ inline TileWalk(int total_, int gm_, int gn_)
@@ -106,7 +109,7 @@ struct TileWalk {
     __device__ inline bool has_next() const { return lin + static_cast<int>(gridDim.x) < total; }
     __device__ inline void coords(bool next, int& tm, int& tn) const
     {
-        xcd_tile(next ? lin + static_cast<int>(gridDim.x) : lin, total, gm, gn, 8, tm, tn);
+        xcd_tile(next ? lin + static_cast<int>(gridDim.x) : lin, total, gm, gn, RLK_WALK_PATCH, tm, tn);
     }
     __device__ inline void advance() { lin += static_cast<int>(gridDim.x); }
 };
