@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "f40ed3feaf6d5501",
-    "measured_at_commit": "32aaa94",
+    "kernel_source_sha16": "c7e4a69fcbbc338b",
+    "measured_at_commit": "0fbcaba",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 51445453564,
-        "linear_logp_dz_kernel": 1963404015,
-        "linear_logp_dh_kernel": 1837065263,
-        "linear_logp_dw_kernel": 2158194980,
+        "linear_logp_fwd_kernel": 51808433484,
+        "linear_logp_dz_kernel": 1970161255,
+        "linear_logp_dh_kernel": 1840708689,
+        "linear_logp_dw_kernel": 2157986636,
     },
 }
 
