@@ -113,7 +113,13 @@ struct WideIO {
     int rows, K;
     bool vec;
 
-    __device__ inline void init(const WideOperand& op, int K_)
+    // FAST (see fast_ok): every group is one aligned 4-element load, no per-element checks.
+    static __device__ inline bool fast_ok(const WideOperand& op, int K_)
+    {
+        return op.vec && K_ % kWBK == 0 && (!KMAJOR || (op.rows & 3) == 0);
+    }
+
+    __device__ inline void init(const WideOperand& op, int K_, bool fast)
     {
         base = op.base;
         rows = op.rows;
@@ -125,7 +131,9 @@ struct WideIO {
             const int idx = g * kThreads + static_cast<int>(threadIdx.x);
             if (KMAJOR) {
                 const int line = idx >> 6, r = (idx & 63) * 4;
-                off[g] = static_cast<int64_t>(line) * op.ld + (r < rows ? r : rows - 1);
+                // past the valid rows: the last valid element, or (FAST) the last valid group
+                const int last = fast ? rows - 4 : rows - 1;
+                off[g] = static_cast<int64_t>(line) * op.ld + (r < rows ? r : last);
             } else {
                 const int row = idx >> 2, k = (idx & 3) * 4;
                 off[g] = static_cast<int64_t>(row < rows ? row : rows - 1) * op.ld + k;
@@ -133,8 +141,10 @@ struct WideIO {
         }
     }
 
+    template <bool FAST>
     __device__ inline f32x4_t load(int kt, int g) const
     {
+        if (FAST) return E::get4(base, off[g] + kt * step);
         const int idx = g * kThreads + static_cast<int>(threadIdx.x);
         f32x4_t v{0.f, 0.f, 0.f, 0.f};
         if (KMAJOR) {
@@ -228,19 +238,29 @@ struct WideGemm {
     __device__ static inline void run(const WideOperand& A, const WideOperand& B, int K,
                                       f32x16_t (&acc)[kTM][kTN], char* smem_c)
     {
+        if (IOA::fast_ok(A, K) && IOB::fast_ok(B, K))  // uniform
+            run_impl<true>(A, B, K, acc, smem_c);
+        else
+            run_impl<false>(A, B, K, acc, smem_c);
+    }
+
+    template <bool FAST>
+    __device__ static inline void run_impl(const WideOperand& A, const WideOperand& B, int K,
+                                           f32x16_t (&acc)[kTM][kTN], char* smem_c)
+    {
         float* smem = reinterpret_cast<float*>(smem_c);
         IOA la;
         IOB lb;
-        la.init(A, K);
-        lb.init(B, K);
+        la.init(A, K, FAST);
+        lb.init(B, K, FAST);
         const int wave = threadIdx.x >> 6;
         const int wm = wave / kWN, wn = wave % kWN;
         const int nk = (K + kWBK - 1) / kWBK;
         f32x4_t ra[2], rb[2];
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-            ra[g] = la.load(0, g);
-            rb[g] = lb.load(0, g);
+            ra[g] = la.template load<FAST>(0, g);
+            rb[g] = lb.template load<FAST>(0, g);
         }
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
@@ -250,8 +270,8 @@ struct WideGemm {
         if (nk > 1) {  // uniform
 #pragma unroll
             for (int g = 0; g < 2; ++g) {
-                ra[g] = la.load(1, g);
-                rb[g] = lb.load(1, g);
+                ra[g] = la.template load<FAST>(1, g);
+                rb[g] = lb.template load<FAST>(1, g);
             }
         }
         __syncthreads();
@@ -271,8 +291,8 @@ struct WideGemm {
             if (kt + 2 < nk) {
 #pragma unroll
                 for (int g = 0; g < 2; ++g) {
-                    ra[g] = la.load(kt + 2, g);
-                    rb[g] = lb.load(kt + 2, g);
+                    ra[g] = la.template load<FAST>(kt + 2, g);
+                    rb[g] = lb.template load<FAST>(kt + 2, g);
                 }
             }
             frags(cur, wm, wn, 1, fa1, fb1);

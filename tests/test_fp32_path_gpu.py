@@ -32,6 +32,7 @@ def op():
     ((3, 200), 130, 1000, torch.float32, True, 0.7, True, 1e-5),    # 3 token blocks x 4 vocab tiles, ragged
     ((700,), 515, 777, torch.float32, False, 1.0, False, 2e-5),     # odd H: element-wise loads, 3 H tiles
     ((300,), 260, 520, torch.bfloat16, True, 1.0, True, 1e-3),      # 16-bit, H % 8 != 0, several tiles
+    ((2048,), 512, 8192, torch.float32, True, 0.9, True, 2e-5),     # 8 x 32 x 2 tiles, dH in 8 vocab parts
 ])
 def test_forward_backward_match_oracle(dev, op, lead, h, v, dtype, bias, temp, ign, atol):
     g = torch.Generator().manual_seed(h + v)

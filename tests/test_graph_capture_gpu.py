@@ -9,15 +9,17 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def test_forward_backward_replay_in_a_hip_graph():
+@pytest.mark.parametrize("dt,tdtype,h", [(0, torch.bfloat16, 256),   # 16-bit MFMA kernels
+                                         (2, torch.float32, 250)])   # fp32 matrix-core kernels, odd H
+def test_forward_backward_replay_in_a_hip_graph(dt, tdtype, h):
     from rl_kernel_amd import _native
 
     lib = _native.load()
     dev = torch.device("cuda:0")
-    n, h, v, dt = 700, 256, 3000, 0  # bf16; ragged token and vocab tails
+    n, v = 700, 3000  # ragged token and vocab tails
     g = torch.Generator(device=dev).manual_seed(5)
-    hidden = torch.randn(n, h, device=dev, generator=g).to(torch.bfloat16)
-    weight = (torch.randn(v, h, device=dev, generator=g) * 0.06).to(torch.bfloat16)
+    hidden = torch.randn(n, h, device=dev, generator=g).to(tdtype)
+    weight = (torch.randn(v, h, device=dev, generator=g) * 0.06).to(tdtype)
     targets = torch.randint(0, v, (n,), device=dev, generator=g)
     targets[::13] = -100
     grad = torch.randn(n, device=dev, generator=g)
@@ -55,7 +57,7 @@ def test_forward_backward_replay_in_a_hip_graph():
         enqueue(side.cuda_stream)
 
     for it in range(3):
-        hidden.copy_(torch.randn(n, h, device=dev, generator=g).to(torch.bfloat16))
+        hidden.copy_(torch.randn(n, h, device=dev, generator=g).to(tdtype))
         grad.copy_(torch.randn(n, device=dev, generator=g))
         graph.replay()
         torch.cuda.synchronize()
