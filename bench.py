@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "c7e4a69fcbbc338b",
-    "measured_at_commit": "0fbcaba",
+    "kernel_source_sha16": "012ea7fa88e01103",
+    "measured_at_commit": "4341033",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 51808433484,
-        "linear_logp_dz_kernel": 1970161255,
-        "linear_logp_dh_kernel": 1840708689,
-        "linear_logp_dw_kernel": 2157986636,
+        "linear_logp_fwd_kernel": 52053158748,
+        "linear_logp_dz_kernel": 1968306809,
+        "linear_logp_dh_kernel": 1843870664,
+        "linear_logp_dw_kernel": 2158486326,
     },
 }
 
