@@ -1354,6 +1354,24 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
     return 0;
 }
 
+// One forward contraction launch: a.row_blocks x a.n_split workgroups of the given variant.
+template <class T, bool GENERAL>
+int launch_fwd_as(const FwdArgs& a, hipStream_t stream)
+{
+    using G = TileGemm<T, false, false, kBK>;
+    if (int rc = set_smem(linear_logp_fwd_kernel<T, kBK, GENERAL>, G::kSmemBytes)) return rc;
+    hipLaunchKernelGGL((linear_logp_fwd_kernel<T, kBK, GENERAL>), dim3(a.row_blocks * a.n_split),
+                       dim3(kThreads), G::kSmemBytes, stream, a);
+    return 0;
+}
+
+template <bool GENERAL>
+int launch_fwd(const FwdArgs& a, int32_t dtype, hipStream_t stream)
+{
+    return dtype == RLK_DTYPE_BF16 ? launch_fwd_as<Bf16, GENERAL>(a, stream)
+                                   : launch_fwd_as<F16, GENERAL>(a, stream);
+}
+
 // A second head over the same hidden states and targets (a frozen reference model).
 struct SecondHead {
     const void* weight;
@@ -1600,38 +1618,19 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
                                            dtype, temperature, stream))
                 return rc;
     }
-    using G = TileGemm<Bf16, false, false, kBK>;  // same LDS footprint for f16
     if (mfma && plan.n_fast > 0) {
         a.n_split = plan.n_fast;
         a.split_lo = 0;
         a.tile_lo = 0;
         a.vtiles = plan.fast_tiles;
-        const int grid = a.row_blocks * a.n_split;
-        if (dtype == RLK_DTYPE_BF16) {
-            if (int rc = set_smem(linear_logp_fwd_kernel<Bf16, kBK, false>, G::kSmemBytes)) return rc;
-            hipLaunchKernelGGL((linear_logp_fwd_kernel<Bf16, kBK, false>), dim3(grid), dim3(kThreads),
-                               G::kSmemBytes, stream, a);
-        } else {
-            if (int rc = set_smem(linear_logp_fwd_kernel<F16, kBK, false>, G::kSmemBytes)) return rc;
-            hipLaunchKernelGGL((linear_logp_fwd_kernel<F16, kBK, false>), dim3(grid), dim3(kThreads),
-                               G::kSmemBytes, stream, a);
-        }
+        if (int rc = launch_fwd<false>(a, dtype, stream)) return rc;
     }
     if (mfma && plan.n_gen > 0) {
         a.n_split = plan.n_gen;
         a.split_lo = plan.n_fast;
         a.tile_lo = plan.fast_tiles;
         a.vtiles = plan.gen_tiles;
-        const int grid = a.row_blocks * a.n_split;
-        if (dtype == RLK_DTYPE_BF16) {
-            if (int rc = set_smem(linear_logp_fwd_kernel<Bf16, kBK, true>, G::kSmemBytes)) return rc;
-            hipLaunchKernelGGL((linear_logp_fwd_kernel<Bf16, kBK, true>), dim3(grid), dim3(kThreads),
-                               G::kSmemBytes, stream, a);
-        } else {
-            if (int rc = set_smem(linear_logp_fwd_kernel<F16, kBK, true>, G::kSmemBytes)) return rc;
-            hipLaunchKernelGGL((linear_logp_fwd_kernel<F16, kBK, true>), dim3(grid), dim3(kThreads),
-                               G::kSmemBytes, stream, a);
-        }
+        if (int rc = launch_fwd<true>(a, dtype, stream)) return rc;
     }
     if (int rc = check_launch("linear_logp_fwd_kernel launch failed")) return rc;
 
