@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "012ea7fa88e01103",
-    "measured_at_commit": "4341033",
+    "kernel_source_sha16": "467b861792cabe44",
+    "measured_at_commit": "e2e3422",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 52053158748,
-        "linear_logp_dz_kernel": 1968306809,
-        "linear_logp_dh_kernel": 1843870664,
-        "linear_logp_dw_kernel": 2158486326,
+        "linear_logp_fwd_kernel": 51391683766,
+        "linear_logp_dz_kernel": 1965205252,
+        "linear_logp_dh_kernel": 1837397216,
+        "linear_logp_dw_kernel": 2159409934,
     },
 }
 
