@@ -90,8 +90,11 @@ REFERENCE_PUBLISHED_H100 = {
 
 
 def kernel_source_sha16() -> str:
+    """Digest of the device-code sources (kernels and their headers; the PyTorch binding is host
+    code only)."""
     m = hashlib.sha256()
-    for path in sorted(glob.glob(os.path.join(ROOT, "rl-kernel_amd", "csrc", "*"))):
+    csrc = os.path.join(ROOT, "rl-kernel_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(csrc, "*.hip")) + glob.glob(os.path.join(csrc, "*.hpp"))):
         with open(path, "rb") as fh:
             m.update(os.path.basename(path).encode())
             m.update(fh.read())

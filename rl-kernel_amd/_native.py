@@ -3,6 +3,7 @@
 from __future__ import annotations
 
 import ctypes
+import functools
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -107,3 +108,21 @@ def check(rc: int, what: str) -> None:
     if rc == -2:
         raise NotImplementedError(f"{what}: {msg}")
     raise RuntimeError(f"{what}: {msg} (code {rc})")
+
+
+def on_tensor_device(fn):
+    """Run ``fn`` with the GPU of its first CUDA tensor argument as the current device: the C ABI
+    launches on a stream handle and HIP requires that stream's device to be current, which is not
+    a given on a host with several GPUs."""
+
+    @functools.wraps(fn)
+    def guarded(*args, **kwargs):
+        import torch
+
+        for a in args:
+            if isinstance(a, torch.Tensor) and a.is_cuda:
+                with torch.cuda.device(a.device):
+                    return fn(*args, **kwargs)
+        return fn(*args, **kwargs)
+
+    return guarded

@@ -7,6 +7,7 @@
 #include <torch/extension.h>
 
 #include <ATen/hip/HIPContext.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 
 #include <vector>
 
@@ -37,6 +38,8 @@ std::vector<at::Tensor> fused_linear_logp(at::Tensor hidden, at::Tensor weight, 
 {
     TORCH_CHECK(hidden.dim() == 2 && weight.dim() == 2, "hidden and weight must be 2D tensors");
     TORCH_CHECK(hidden.is_cuda() && weight.is_cuda(), "hidden and weight must be CUDA tensors");
+    // allocations and launches below go to the tensors' GPU, whichever device is current
+    const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(hidden.device());
     TORCH_CHECK(weight.size(1) == hidden.size(1), "hidden/weight hidden-dim mismatch");
     TORCH_CHECK(target.numel() == hidden.size(0), "target must have one id per token: expected ",
                 hidden.size(0), " (hidden rows), got ", target.numel());
@@ -88,6 +91,7 @@ at::Tensor scan_into(const at::Tensor& logits, const at::Tensor& token_ids,
     TORCH_CHECK(in_dt == RLK_DTYPE_BF16 || in_dt == RLK_DTYPE_F16 || in_dt == RLK_DTYPE_F32,
                 "logits dtype must be float32, float16 or bfloat16");
     TORCH_CHECK(out_dt >= 0, "output dtype must be float64, float32, float16, or bfloat16");
+    const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(logits.device());
     auto lg = logits.contiguous();
     auto ids = token_ids.contiguous();
     at::Tensor idx;

@@ -34,6 +34,7 @@ def _require_gpu(name: str) -> None:
     _native.load()
 
 
+@_native.on_tensor_device
 def grpo_from_logp_raw(cur, old, ref, adv, mask, *, clip_eps, beta, want_grad, want_terms=False,
                        upstream=None):
     """One launch set of the epilogue; returns ``(out3, ratio, kl_terms, d_cur, d_kl)``."""
@@ -97,6 +98,7 @@ class _GRPOFromLogpFunction(torch.autograd.Function):
         return grad.to(ctx.cur_dtype), None, None, None, None, None, None
 
 
+@_native.on_tensor_device
 def group_advantages(rewards: torch.Tensor, *, samples_per_prompt: Optional[int] = None,
                      group_boundaries=None, eps: float = 1e-6) -> torch.Tensor:
     """Group-normalised advantages on the GPU; argument policy of

@@ -22,6 +22,7 @@ from . import linear_logp as LL
 IGNORE_INDEX = -100
 
 
+@_native.on_tensor_device
 def fused_linear_logp_grpo_forward(hidden_2d, weight, target_1d, bias, old, ref, adv, mask, *,
                                    seq_len: int, clip_eps: float, beta: float,
                                    temperature: float = 1.0, ignore_index: Optional[int] = None,

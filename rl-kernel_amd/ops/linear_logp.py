@@ -88,6 +88,7 @@ def _warn_if_wide_path(hidden_2d: torch.Tensor, weight: torch.Tensor) -> None:
             weight.size(0))
 
 
+@_native.on_tensor_device
 def fused_linear_logp_forward(
     hidden_2d: torch.Tensor,
     weight: torch.Tensor,
@@ -130,6 +131,7 @@ def fused_linear_logp_forward(
     return logp, lse, err
 
 
+@_native.on_tensor_device
 def fused_linear_logp_forward_pair(
     hidden_2d: torch.Tensor,
     weight: torch.Tensor,
@@ -174,6 +176,7 @@ def fused_linear_logp_forward_pair(
     return (*outs, err)
 
 
+@_native.on_tensor_device
 def fused_norm_linear_logp_forward(
     x_2d: torch.Tensor,
     gain: torch.Tensor,
@@ -213,6 +216,7 @@ def fused_norm_linear_logp_forward(
     return logp, lse, err
 
 
+@_native.on_tensor_device
 def fused_norm_linear_logp_backward(
     grad_logp: torch.Tensor,
     x_2d: torch.Tensor,
@@ -259,6 +263,7 @@ def fused_norm_linear_logp_backward(
     return d_x, d_gain, d_weight, d_bias
 
 
+@_native.on_tensor_device
 def fused_linear_logp_backward(
     grad_logp: torch.Tensor,
     hidden_2d: torch.Tensor,

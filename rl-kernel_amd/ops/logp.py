@@ -26,6 +26,7 @@ def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+@_native.on_tensor_device
 def logp_from_logits(logits_2d: torch.Tensor, ids_1d: torch.Tensor, output_1d: torch.Tensor,
                      row_indices: Optional[torch.Tensor] = None,
                      lse_out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -174,9 +175,10 @@ class _LogpFromLogitsFunction(torch.autograd.Function):
         coeff = grad_out.reshape(-1).to(torch.float32).contiguous()
         grad = torch.empty_like(logits_2d)
         n, v = logits_2d.shape
-        rc = lib.rlk_logp_from_logits_bwd(logits_2d.data_ptr(), _IN[logits_2d.dtype],
-                                          ids_1d.data_ptr(), lse.data_ptr(), coeff.data_ptr(),
-                                          grad.data_ptr(), n, v, _stream(logits_2d.device))
+        with torch.cuda.device(logits_2d.device):
+            rc = lib.rlk_logp_from_logits_bwd(logits_2d.data_ptr(), _IN[logits_2d.dtype],
+                                              ids_1d.data_ptr(), lse.data_ptr(), coeff.data_ptr(),
+                                              grad.data_ptr(), n, v, _stream(logits_2d.device))
         _native.check(rc, "rlk_logp_from_logits_bwd")
         return grad.view(ctx.logits_shape), None
 
@@ -196,10 +198,11 @@ class _LogpPairFromLogitsFunction(torch.autograd.Function):
         ref_out = torch.empty(n, device=logits.device, dtype=torch.float32)
         lse = torch.empty(n, device=logits.device, dtype=torch.float32)
         if n > 0:
-            rc = _native.load().rlk_logp_from_logits_pair(
-                logits_2d.data_ptr(), ref_2d.data_ptr(), _IN[logits_2d.dtype], ids_1d.data_ptr(),
-                out.data_ptr(), ref_out.data_ptr(), _OUT[torch.float32], lse.data_ptr(), None, None,
-                n, n, v, _stream(logits_2d.device))
+            with torch.cuda.device(logits_2d.device):
+                rc = _native.load().rlk_logp_from_logits_pair(
+                    logits_2d.data_ptr(), ref_2d.data_ptr(), _IN[logits_2d.dtype], ids_1d.data_ptr(),
+                    out.data_ptr(), ref_out.data_ptr(), _OUT[torch.float32], lse.data_ptr(), None, None,
+                    n, n, v, _stream(logits_2d.device))
             _native.check(rc, "rlk_logp_from_logits_pair")
         ctx.save_for_backward(logits_2d, ids_1d, lse)
         ctx.logits_shape = logits.shape

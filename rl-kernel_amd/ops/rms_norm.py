@@ -15,6 +15,7 @@ from ..platform import logger
 from .linear_logp import _DTYPES, _aligned_contiguous, _ptr, _stream
 
 
+@_native.on_tensor_device
 def rmsnorm_forward(x_2d: torch.Tensor, gain: torch.Tensor, eps: float) -> torch.Tensor:
     """Raw launch: normalised rows in the dtype of ``x_2d`` ([N, H] contiguous, gain [H] same dtype)."""
     out = torch.empty_like(x_2d)
@@ -27,6 +28,7 @@ def rmsnorm_forward(x_2d: torch.Tensor, gain: torch.Tensor, eps: float) -> torch
     return out
 
 
+@_native.on_tensor_device
 def rmsnorm_backward(x_2d: torch.Tensor, gain: torch.Tensor, eps: float, d_out: torch.Tensor):
     """Raw launch: ``(d_x [N, H] in the dtype of x, d_gain [H] fp32)``."""
     lib = _native.load()
