@@ -506,15 +506,18 @@ struct DhArgs {
 // before the first use, then added and stored.  FULL (the tile lies inside the chunk and inside
 // H): addresses are a uniform tile origin plus a 32-bit lane offset and no predicates are needed;
 // otherwise rows and columns are clamped for the reads and predicated for the stores.
+// The tile covers hidden columns [h0, h0 + 256) and owns those from h_min on (h_min > h0 for the
+// last tile of a persistent walk when H is not a multiple of 256: it is shifted back to end at H
+// and must leave the columns of its left neighbour alone).
 template <class T, bool FULL>
 __device__ inline void dh_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const DhArgs& a, int tt,
-                                        int ht, float* acc_dst, bool first, bool last)
+                                        int h0, int h_min, float* acc_dst, bool first, bool last)
 {
     constexpr int TM = kTM, TN = kTN;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
-    const int tok0 = tt * 256, h0 = ht * 256;
+    const int tok0 = tt * 256;
     const float oscale = a.scales[1];
     const int hbase = h0 + wm * (TM * 32) + 4 * (lane >> 5);  // + i * 32 + 8 * q
     const uint32_t ldh = static_cast<uint32_t>(a.H);
@@ -554,7 +557,7 @@ __device__ inline void dh_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const D
                           acc[i][j][q * 4 + 3]};
                 v += old[i][q];
                 const size_t uni = static_cast<size_t>(j * 32) * ldh + (i * 32 + 8 * q);  // uniform
-                if (FULL || (tok_ok && h < a.H)) {  // H % 8 == 0: a quad is all-in or all-out
+                if (FULL || (tok_ok && h >= h_min && h < a.H)) {  // H % 8 == 0: a quad is all-in or all-out
                     if (last) {
                         u32x2_t pk{T::pack2(v.x * oscale, v.y * oscale), T::pack2(v.z * oscale, v.w * oscale)};
                         if (FULL)
@@ -574,19 +577,19 @@ __device__ inline void dh_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const D
 
 // Returns whether the tile was full (then every wavefront issued all its stores unconditionally).
 template <class T>
-__device__ inline bool dh_epilogue(const f32x16_t (&acc)[kTM][kTN], const DhArgs& a, int tt, int ht,
-                                   float* acc_dst, bool first, bool last)
+__device__ inline bool dh_epilogue(const f32x16_t (&acc)[kTM][kTN], const DhArgs& a, int tt, int h0,
+                                   int h_min, float* acc_dst, bool first, bool last)
 {
-    const bool full = tt * 256 + 256 <= a.tok_valid && ht * 256 + 256 <= a.H;  // uniform
+    const bool full = tt * 256 + 256 <= a.tok_valid && h0 + 256 <= a.H && h_min == h0;  // uniform
     if (full)
-        dh_epilogue_impl<T, true>(acc, a, tt, ht, acc_dst, first, last);
+        dh_epilogue_impl<T, true>(acc, a, tt, h0, h_min, acc_dst, first, last);
     else
-        dh_epilogue_impl<T, false>(acc, a, tt, ht, acc_dst, first, last);
+        dh_epilogue_impl<T, false>(acc, a, tt, h0, h_min, acc_dst, first, last);
     return full;
 }
 
-// CHAIN (needs ksplit == 1, H a multiple of 256, v_valid a multiple of BK and >= 2 BK): the
-// workgroup walks its tiles through one pipeline.
+// CHAIN (needs ksplit == 1, H >= 256, v_valid a multiple of BK and >= 2 BK): the workgroup walks
+// its tiles through one pipeline.
 template <class T, int BK, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
 {
@@ -599,7 +602,9 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
         if (!walk.valid()) return;
         int tt, ht;
         walk.coords(false, tt, ht);
-        auto w_origin = [&](int h) { return a.weight + static_cast<int64_t>(h) * 256; };
+        // first hidden column of h tile `h`: the last tile is shifted back so that it ends at H
+        auto h_col = [&](int h) { return min(h * 256, a.H - 256); };
+        auto w_origin = [&](int h) { return a.weight + h_col(h); };
         auto z_origin = [&](int t) { return a.dz + static_cast<int64_t>(t) * 256 * a.ldz; };
         typename Dtl::Stream st;
         bool counted = false;
@@ -612,7 +617,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
             // a full tile's epilogue issues kTM * kTN * 4 unconditional stores per wavefront
             Dtl::template tile<true, kTM * kTN * 2>(st, w_origin(nht), z_origin(ntt), acc, smem, counted);
             if (more) Dtl::fetch_ahead(st, smem);
-            counted = dh_epilogue<T>(acc, a, tt, ht, a.acc, a.first != 0, a.last != 0);
+            counted = dh_epilogue<T>(acc, a, tt, h_col(ht), ht * 256, a.acc, a.first != 0, a.last != 0);
             if (!more) break;
             walk.advance();
             tt = ntt;
@@ -651,7 +656,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
         zero_acc(acc);
         Gemm::run(A, B, kn, acc, smem);
         if (empty_part) zero_acc(acc);  // uniform: this part's slot must hold zeros
-        dh_epilogue<T>(acc, a, tt, ht, acc_dst, first, last);
+        dh_epilogue<T>(acc, a, tt, h0, h0, acc_dst, first, last);
     }
 }
 
@@ -700,14 +705,16 @@ struct DwArgs {
 // per 32-row group): the 16 reads of a batch are issued before the first use.  FULL (the tile lies
 // inside the piece and inside H): a uniform tile origin plus a 32-bit lane offset, no predicates;
 // otherwise clamped reads and predicated stores.
+// The tile covers hidden columns [h0, h0 + 256) and owns those from h_min on (see dh_epilogue_impl).
 template <bool FULL>
-__device__ inline void dw_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const DwArgs& a, int vt, int ht)
+__device__ inline void dw_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const DwArgs& a, int vt, int h0,
+                                        int h_min)
 {
     constexpr int TM = kTM, TN = kTN;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
-    const int v0 = vt * 256, h0 = ht * 256;
+    const int v0 = vt * 256;
     const float oscale = a.scales[1];
     const int hbase = h0 + wm * (TM * 32) + 4 * (lane >> 5);  // + i * 32 + 8 * q
     const uint32_t ldw = static_cast<uint32_t>(a.H);
@@ -747,7 +754,7 @@ __device__ inline void dw_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const D
                 if (FULL) {
                     char* rowp = tile + (static_cast<size_t>(j * 32) * ldw + (i * 32 + 8 * q)) * 4u;
                     *reinterpret_cast<f32x4_t*>(rowp + lane_el * 4u) = val;
-                } else if (v_ok && h < a.H) {  // H % 8 == 0: a quad is all-in or all-out
+                } else if (v_ok && h >= h_min && h < a.H) {  // H % 8 == 0: a quad is all-in or all-out
                     *reinterpret_cast<f32x4_t*>(a.dw + vrow + h) = val;
                 }
             }
@@ -755,18 +762,19 @@ __device__ inline void dw_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const D
 }
 
 // Returns whether the tile was full (then every wavefront issued all its stores unconditionally).
-__device__ inline bool dw_epilogue(const f32x16_t (&acc)[kTM][kTN], const DwArgs& a, int vt, int ht)
+__device__ inline bool dw_epilogue(const f32x16_t (&acc)[kTM][kTN], const DwArgs& a, int vt, int h0,
+                                   int h_min)
 {
-    const bool full = vt * 256 + 256 <= a.v_valid && ht * 256 + 256 <= a.H;  // uniform
+    const bool full = vt * 256 + 256 <= a.v_valid && h0 + 256 <= a.H && h_min == h0;  // uniform
     if (full)
-        dw_epilogue_impl<true>(acc, a, vt, ht);
+        dw_epilogue_impl<true>(acc, a, vt, h0, h_min);
     else
-        dw_epilogue_impl<false>(acc, a, vt, ht);
+        dw_epilogue_impl<false>(acc, a, vt, h0, h_min);
     return full;
 }
 
-// CHAIN (needs H a multiple of 256, tok_valid a multiple of BK and >= 2 BK): the workgroup walks
-// its tiles through one pipeline.
+// CHAIN (needs H >= 256, tok_valid a multiple of BK and >= 2 BK): the workgroup walks its tiles
+// through one pipeline.
 template <class T, int BK, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
 {
@@ -778,9 +786,11 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
     int vt, ht;
     walk.coords(false, vt, ht);
     f32x16_t acc[kTM][kTN];
-    auto h_origin = [&](int h) { return a.hidden + static_cast<int64_t>(h) * 256; };  // M rows
     auto z_origin = [&](int v) { return a.dz + static_cast<int64_t>(v) * 256; };      // N rows
     if constexpr (CHAIN) {
+        // first hidden column of h tile `h`: the last tile is shifted back so that it ends at H
+        auto h_col = [&](int h) { return min(h * 256, a.H - 256); };
+        auto h_origin = [&](int h) { return a.hidden + h_col(h); };  // M rows
         typename Dtl::Stream st;
         bool counted = false;
         Dtl::begin(st, Operand{h_origin(ht), a.H, 256}, Operand{z_origin(vt), a.ldz, 256}, a.tok_valid, smem);
@@ -792,7 +802,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
             // a full tile's epilogue issues kTM * kTN * 4 unconditional stores per wavefront
             Dtl::template tile<true, kTM * kTN * 2>(st, h_origin(nht), z_origin(nvt), acc, smem, counted);
             if (more) Dtl::fetch_ahead(st, smem);
-            counted = dw_epilogue(acc, a, vt, ht);
+            counted = dw_epilogue(acc, a, vt, h_col(ht), ht * 256);
             if (!more) break;
             walk.advance();
             vt = nvt;
@@ -801,11 +811,11 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
         Dtl::end(st);
     } else {
         for (;;) {
-            Operand A{h_origin(ht), a.H, min(256, a.H - ht * 256)};
+            Operand A{a.hidden + static_cast<int64_t>(ht) * 256, a.H, min(256, a.H - ht * 256)};
             Operand B{z_origin(vt), a.ldz, 256};
             zero_acc(acc);
             Gemm::run(A, B, a.tok_valid, acc, smem);
-            dw_epilogue(acc, a, vt, ht);
+            dw_epilogue(acc, a, vt, ht * 256, ht * 256);
             if (!walk.has_next()) break;
             walk.advance();
             walk.coords(false, vt, ht);
@@ -1314,7 +1324,7 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             }
             if (dh) {
                 const int tiles = tok_tiles * h_tiles;
-                if (RLK_CHAIN_DH && p.ksplit == 1 && H % 256 == 0 && v_valid % kBK == 0 && v_valid >= 2 * kBK) {
+                if (RLK_CHAIN_DH && p.ksplit == 1 && H >= 256 && v_valid % kBK == 0 && v_valid >= 2 * kBK) {
                     hipLaunchKernelGGL((linear_logp_dh_kernel<T, kBK, true>),
                                        dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kChainSmem,
                                        stream, h);
@@ -1332,7 +1342,7 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             }
             if (c.d_weight) {
                 const int tiles = v_tiles * h_tiles;
-                if (RLK_CHAIN_DW && H % 256 == 0 && tok_valid % kBK == 0 && tok_valid >= 2 * kBK)
+                if (RLK_CHAIN_DW && H >= 256 && tok_valid % kBK == 0 && tok_valid >= 2 * kBK)
                     hipLaunchKernelGGL((linear_logp_dw_kernel<T, kBK, true>),
                                        dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kChainSmem,
                                        stream, d);

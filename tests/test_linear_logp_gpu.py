@@ -472,6 +472,33 @@ def test_element_offsets_beyond_32_bits(dev, n, h, v):
 
 
 @pytest.mark.parametrize("n,h,v,dtype,budget", [
+    (1024, 320, 2048, torch.bfloat16, 1 << 20),    # 2 chunks x 2 pieces, last h tile 64 wide
+    (1024, 896, 2048, torch.float16, 1 << 20),     # last h tile 128 wide (H = 3.5 tiles)
+    (768, 520, 3072, torch.bfloat16, 0),           # one block, H not a multiple of the K step
+])
+def test_ragged_hidden_tile_in_the_persistent_backward(dev, n, h, v, dtype, budget):
+    """H >= 256 that is not a multiple of 256: the persistent dH / dW walks shift their last h tile
+    back so that it ends at H and store only the columns it owns; with several vocab pieces and
+    token chunks every store mode (write, read-add-write, final 16-bit write) sees such a tile."""
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    hidden, weight, _, tgt, grad = make(11, (n,), h, v, dtype, False, 0.05)
+    r_dh, r_dw, _ = O.linear_logp_backward(grad, hidden, weight, tgt, None, ignore_index=-100)
+    hd, wd, td = hidden.to(dev), weight.to(dev), tgt.to(dev)
+    _, lse, _ = LL.fused_linear_logp_forward(hd, wd, td, ignore_index=-100)
+    dh, dw, _ = LL.fused_linear_logp_backward(grad.to(dev), hd, wd, td, lse, ignore_index=-100,
+                                              dz_budget_bytes=budget)
+    assert rel(dh, r_dh) < GRAD_REL and rel(dw, r_dw) < GRAD_REL
+    # column by column: the shifted tile must neither skip nor double-count a column
+    for lo in range(0, h, 64):
+        assert rel(dh[:, lo:lo + 64], r_dh[:, lo:lo + 64]) < GRAD_REL, lo
+        assert rel(dw[:, lo:lo + 64], r_dw[:, lo:lo + 64]) < GRAD_REL, lo
+    dh2, dw2, _ = LL.fused_linear_logp_backward(grad.to(dev), hd, wd, td, lse, ignore_index=-100,
+                                                dz_budget_bytes=budget)
+    assert torch.equal(dh, dh2) and torch.equal(dw, dw2)
+
+
+@pytest.mark.parametrize("n,h,v,dtype,budget", [
     (300, 64, 40000, torch.bfloat16, 0),           # one piece, dH range cut into parts
     (513, 128, 70001, torch.float16, 16 << 20),    # several pieces, ragged last piece and K tail
     (1024, 256, 32868, torch.bfloat16, 32 << 20),  # 100-row last piece: two of four parts stay empty
