@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "c1ab68fb7099b375",
-    "measured_at_commit": "163301a",
+    "kernel_source_sha16": "25add9575034c4bf",
+    "measured_at_commit": "35925c1",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 51081630168,
-        "linear_logp_dz_kernel": 1966067403,
-        "linear_logp_dh_kernel": 1840267362,
-        "linear_logp_dw_kernel": 2161265340,
+        "linear_logp_fwd_kernel": 51430051661,
+        "linear_logp_dz_kernel": 1962480064,
+        "linear_logp_dh_kernel": 1841536417,
+        "linear_logp_dw_kernel": 2170045622,
     },
 }
 
