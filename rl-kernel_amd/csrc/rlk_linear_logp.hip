@@ -1021,10 +1021,28 @@ struct BwdPlan {
 // Measured on MI355X with wall-clock stamps inside the kernels, one K step (256 x 256 x 64) takes
 // about 1.56 us in all three kernels; the dZ epilogue (exp + 16-bit store) 4.4 us = 3 steps, the
 // fp32 read-modify-write of a dH or dW tile 13 - 14 us = 9 steps.
+// Few tokens or a narrow hidden dimension: a dH launch of at most 128 tiles over a long vocab range
+// is cut into parts that run side by side (fp32 slots, added up in slot order afterwards).
+inline int dh_parts(int64_t ct, int64_t pt, int64_t ht)
+{
+    const int64_t tiles = ct * ht;
+    int parts = 1;
+    if (tiles <= 128 && pt >= 32) {
+        int64_t lim = 256 / tiles;
+        if (lim > pt / 16) lim = pt / 16;
+        if (lim > 8) lim = 8;
+        while (parts * 2 <= lim) parts *= 2;
+    }
+    return parts;
+}
+
 inline int64_t block_cost(int64_t ct, int64_t pt, int64_t ht, int64_t hk)
 {
     const int64_t dz = (ct * pt + 255) / 256 * (hk + 3);
-    const int64_t dh = (ct * ht + 255) / 256 * (4 * pt + 9);
+    const int parts = dh_parts(ct, pt, ht);
+    // split launch: every part is a workgroup of its own; the slot reduction costs about 10 steps
+    const int64_t dh = parts > 1 ? (ct * ht * parts + 255) / 256 * (4 * pt / parts + 9) + 10
+                                 : (ct * ht + 255) / 256 * (4 * pt + 9);
     const int64_t dw = (pt * ht + 255) / 256 * (4 * ct + 9);
     return dz + dh + dw;
 }
@@ -1097,14 +1115,7 @@ BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
     p.acc_off = p.dz_off + align_up(p.dz_bytes, 256);
     // Few tokens: the dH launch has fewer tiles than the chip has CUs but a long vocab range, so
     // the range is cut into parts that run side by side and are added up in a fixed order.
-    p.ksplit = 1;
-    const int64_t dh_tiles = best_ct * ht;
-    if (dh_tiles <= 128 && best_pt >= 32) {
-        int64_t lim = 256 / dh_tiles;
-        if (lim > best_pt / 16) lim = best_pt / 16;
-        if (lim > 8) lim = 8;
-        while (p.ksplit * 2 <= lim) p.ksplit *= 2;
-    }
+    p.ksplit = dh_parts(best_ct, best_pt, ht);
     p.part_bytes = p.ksplit > 1 ? static_cast<size_t>(p.ksplit) * p.tok_chunk * H * 4 : 0;
     p.part_off = p.acc_off + align_up(p.acc_bytes, 256);
     // per-token-tile column sums of the dZ block (d_bias): 1 KiB per dZ tile
