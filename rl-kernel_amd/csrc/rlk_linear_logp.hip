@@ -42,6 +42,7 @@ struct FwdArgs {
     int n_split;     // splits handled by this launch
     int split_lo;    // first slot of the partial arrays this launch writes
     int row_blocks;
+    int patch_rows;  // token blocks of the patch that the workgroups of one XCD cover per round
     int tile_lo;     // first vocab tile of this launch
     int vtiles;      // vocab tiles of this launch
     float scale2;    // log2(e) / temperature
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     int tb, sp;
-    xcd_tile(blockIdx.x, a.row_blocks * a.n_split, a.row_blocks, a.n_split, 8, tb, sp);
+    xcd_tile(blockIdx.x, a.row_blocks * a.n_split, a.row_blocks, a.n_split, a.patch_rows, tb, sp);
     // vocab tiles [t0, t1) of this split: the first (vtiles % n_split) splits take one extra.
     const int base = a.vtiles / a.n_split, extra = a.vtiles % a.n_split;
     const int t0 = a.tile_lo + sp * base + (sp < extra ? sp : extra);
@@ -947,44 +948,53 @@ constexpr int kBK = RLK_BK;
 #define RLK_LDZ_PAD 0
 #endif
 
-// Forward launch plan: a pure function of (N, V, bias present).
-//   fast launch   : full vocab tiles [0, full_tiles) split n_fast ways, no bias
-//   general launch: the remaining tiles (all tiles when there is a bias) split n_gen ways
+// Forward launch plan: a pure function of (N, H, V, which kernels run).
+//   fast launch   : full vocab tiles [0, full_tiles) split n_fast ways
+//   general launch: the ragged last tile (all tiles for the fp32 kernels) split n_gen ways
 struct FwdPlan {
     int row_blocks;
+    int patch_rows;
     int fast_tiles, n_fast;
     int gen_tiles, n_gen;
     int total_splits;
 };
 
-#ifndef RLK_MIN_SPLIT
-#define RLK_MIN_SPLIT 4
-#endif
+// Token blocks per XCD patch.  The 32 workgroups resident on one XCD cover patch_rows token blocks
+// x 32 / patch_rows vocab splits; the hidden blocks of all eight patches in flight (8 x patch_rows
+// x 256 x H x 2 bytes) are re-read for every vocab tile and should stay inside the 256 MB
+// memory-side cache next to the weight tiles: 8 blocks up to H = 4096, 4 up to 8192, 2 beyond
+// (measured at H = 8192 with 16384 tokens and more: 8 blocks 1268 TFLOP/s).
+int patch_rows_for(int H)
+{
+    return H <= 4096 ? 8 : (H <= 8192 ? 4 : 2);
+}
 
-int split_count(int row_blocks, int tiles)
+int split_count(int row_blocks, int tiles, int patch_rows)
 {
     if (tiles <= 0) return 0;
     int s = (512 + row_blocks / 2) / row_blocks;
-    // At least 4 splits when each still gets a long run of tiles: the 32 workgroups resident on
-    // one XCD then form an 8 x 4 (token blocks x splits) patch that fetches 12 distinct operand
-    // streams into its L2 instead of 18 (16 x 2) or 33 (32 x 1).
-    if (s < RLK_MIN_SPLIT && tiles >= RLK_MIN_SPLIT * 16) s = RLK_MIN_SPLIT;
+    // At least 32 / patch_rows splits when each still gets a long run of tiles: the 32 workgroups
+    // resident on one XCD then form a compact (token blocks x splits) patch that fetches 12 distinct
+    // operand streams into its L2 (8 x 4 or 4 x 8) instead of 18 (16 x 2) or 33 (32 x 1).
+    const int want = 32 / patch_rows;
+    if (s < want && tiles >= want * 16) s = want;
     if (s < 1) s = 1;
     if (s > 64) s = 64;
     if (s > tiles) s = tiles;
     return s;
 }
 
-FwdPlan fwd_plan(int64_t N, int64_t V, bool all_general)
+FwdPlan fwd_plan(int64_t N, int H, int64_t V, bool all_general)
 {
     FwdPlan p;
     p.row_blocks = static_cast<int>((N + 255) / 256);
+    p.patch_rows = patch_rows_for(H);
     const int all = static_cast<int>((V + 255) / 256);
     const int full = static_cast<int>(V / 256);
     p.fast_tiles = all_general ? 0 : full;
     p.gen_tiles = all - p.fast_tiles;
-    p.n_fast = split_count(p.row_blocks, p.fast_tiles);
-    p.n_gen = split_count(p.row_blocks, p.gen_tiles);
+    p.n_fast = split_count(p.row_blocks, p.fast_tiles, p.patch_rows);
+    p.n_gen = split_count(p.row_blocks, p.gen_tiles, p.patch_rows);
     p.total_splits = p.n_fast + p.n_gen;
     return p;
 }
@@ -1450,11 +1460,10 @@ extern "C" {
 int rlk_linear_logp_fwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                         size_t* bytes)
 {
-    (void)H;
     (void)dtype;
-    if (!bytes || N <= 0 || V <= 0) return rlk_fail(RLK_ERR_ARG, "bad workspace query");
-    // sized for the larger of the two plans so that one query serves calls with and without bias
-    const int a = fwd_plan(N, V, false).total_splits, b = fwd_plan(N, V, true).total_splits;
+    if (!bytes || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad workspace query");
+    // sized for the larger of the two plans so that one query serves both kinds of kernels
+    const int a = fwd_plan(N, H, V, false).total_splits, b = fwd_plan(N, H, V, true).total_splits;
     *bytes = static_cast<size_t>(3) * (a > b ? a : b) * N * sizeof(float);
     return 0;
 }
@@ -1619,8 +1628,9 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
     a.V = static_cast<int>(V);
     a.vocab_start = vocab_start;
     // the fp32 matrix-core kernels treat every tile as general
-    const FwdPlan plan = fwd_plan(N, V, !mfma);
+    const FwdPlan plan = fwd_plan(N, H, V, !mfma);
     a.row_blocks = plan.row_blocks;
+    a.patch_rows = plan.patch_rows;
     a.part_m = static_cast<float*>(workspace);
     a.part_s = a.part_m + static_cast<size_t>(plan.total_splits) * N;
     a.part_z = a.part_s + static_cast<size_t>(plan.total_splits) * N;
