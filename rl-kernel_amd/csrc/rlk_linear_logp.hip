@@ -964,9 +964,12 @@ struct FwdPlan {
 // x 256 x H x 2 bytes) are re-read for every vocab tile and should stay inside the 256 MB
 // memory-side cache next to the weight tiles: 8 blocks up to H = 4096, 4 up to 8192, 2 beyond
 // (measured at H = 8192 with 16384 tokens and more: 8 blocks 1268 TFLOP/s).
+#ifndef RLK_PATCH8_MAX_H
+#define RLK_PATCH8_MAX_H 4096  // largest hidden size that keeps 8 token blocks per patch
+#endif
 int patch_rows_for(int H)
 {
-    return H <= 4096 ? 8 : (H <= 8192 ? 4 : 2);
+    return H <= RLK_PATCH8_MAX_H ? 8 : (H <= 2 * RLK_PATCH8_MAX_H ? 4 : 2);
 }
 
 int split_count(int row_blocks, int tiles, int patch_rows)
