@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "25add9575034c4bf",
-    "measured_at_commit": "35925c1",
+    "kernel_source_sha16": "316f5378a63c3415",
+    "measured_at_commit": "663f4c5",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 51430051661,
-        "linear_logp_dz_kernel": 1962480064,
-        "linear_logp_dh_kernel": 1841536417,
-        "linear_logp_dw_kernel": 2170045622,
+        "linear_logp_fwd_kernel": 51559718893,
+        "linear_logp_dz_kernel": 1968313923,
+        "linear_logp_dh_kernel": 1848738332,
+        "linear_logp_dw_kernel": 2177399221,
     },
 }
 
