@@ -296,6 +296,22 @@ int rlk_linear_logp_fwd_grpo(const void* hidden, const void* weight, const float
                              int64_t seq_len, float clip_eps, float beta, float* out3, float* ratio,
                              float* kl_terms, float* d_cur, float* d_kl, rlk_stream_t stream);
 
+/* Per-token policy ratio exp(cur - old) and k3 KL exp(ref - cur) - (ref - cur) - 1 of the
+ * logits-fed ratio/KL op, the mask applied to the differences BEFORE the exponentials, so an
+ * inactive position gives ratio 1 and kl 0: the tail of NativeRatioKLOp.forward
+ * (rl_engine/kernels/ops/pytorch/loss/ratio_kl.py:53-58) and of _ratio_kl_fwd_kernel
+ * (rl_engine/kernels/ops/triton/loss/ratio_kl.py:46-60) behind the log-prob scan.  All arrays
+ * fp32 [N] on the device; mask uint8 [N] or NULL (all active).  The backward returns
+ * d_cur = grad_ratio * ratio + grad_kl * (1 - exp(ref - cur)) on active positions, 0 elsewhere
+ * (grad_ratio / grad_kl may be NULL = zero), the coefficient _ratio_kl_bwd_kernel feeds into
+ * the logits gradient (same file :86-122). */
+int rlk_ratio_kl_from_logp(const float* cur_logp, const float* ref_logp, const float* old_logp,
+                           const uint8_t* mask, int64_t N, float* ratio, float* kl,
+                           rlk_stream_t stream);
+int rlk_ratio_kl_from_logp_bwd(const float* cur_logp, const float* ref_logp, const float* old_logp,
+                               const uint8_t* mask, const float* grad_ratio, const float* grad_kl,
+                               int64_t N, float* d_cur, rlk_stream_t stream);
+
 /* Per-group reward normalisation (x - mean_g) / sqrt(max(E_g[x^2] - mean_g^2, eps^2)) over CSR
  * group boundaries (int64 [num_groups + 1], device).  Stands in for
  * NativeGRPOLossOp.group_advantages (rl_engine/kernels/ops/pytorch/loss/grpo_loss.py:53-84) and

@@ -45,6 +45,35 @@ __global__ void grpo_grad_kernel(GrpoArgs a)
     if (a.dkl != nullptr) a.dkl[i] = gk;
 }
 
+// Per-token policy ratio and k3 KL of the logits-fed ratio/KL op: the mask is applied to the
+// log-prob differences before the exponentials, so inactive positions give ratio 1 and kl 0.
+__global__ void ratio_kl_fwd_kernel(const float* cur, const float* ref, const float* old_lp,
+                                    const uint8_t* mask, float* ratio, float* kl, int64_t n)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const bool on = mask == nullptr || mask[i] != 0;
+    const float delta = on ? cur[i] - old_lp[i] : 0.f;
+    const float diff = on ? ref[i] - cur[i] : 0.f;
+    ratio[i] = expf(delta);
+    kl[i] = expf(diff) - diff - 1.f;
+}
+
+// d/d cur of g_ratio * ratio + g_kl * kl: ratio' = ratio, kl' = 1 - exp(ref - cur); 0 when inactive.
+__global__ void ratio_kl_bwd_kernel(const float* cur, const float* ref, const float* old_lp,
+                                    const uint8_t* mask, const float* g_ratio, const float* g_kl,
+                                    float* d_cur, int64_t n)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float g = 0.f;
+    if (mask == nullptr || mask[i] != 0) {
+        if (g_ratio != nullptr) g += g_ratio[i] * expf(cur[i] - old_lp[i]);
+        if (g_kl != nullptr) g += g_kl[i] * (1.f - expf(ref[i] - cur[i]));
+    }
+    d_cur[i] = g;
+}
+
 // One wavefront per group: (x - mean) / sqrt(max(E[x^2] - mean^2, eps^2)).
 __global__ __launch_bounds__(64) void group_advantages_kernel(const float* rewards,
                                                               const int64_t* bounds, float eps,
@@ -127,6 +156,31 @@ int rlk_grpo_loss_from_logp(const float* cur_logp, const float* old_logp, const 
         hipLaunchKernelGGL(grpo_grad_kernel, dim3(static_cast<unsigned>((n_tokens + 255) / 256)),
                            dim3(256), 0, stream, a);
     if (hipGetLastError() != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, "grpo launch failed");
+    return 0;
+}
+
+int rlk_ratio_kl_from_logp(const float* cur_logp, const float* ref_logp, const float* old_logp,
+                           const uint8_t* mask, int64_t N, float* ratio, float* kl, hipStream_t stream)
+{
+    if (!cur_logp || !ref_logp || !old_logp || !ratio || !kl) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (N < 0) return rlk_fail(RLK_ERR_ARG, "bad sizes");
+    if (N == 0) return 0;
+    hipLaunchKernelGGL(ratio_kl_fwd_kernel, dim3(static_cast<unsigned>((N + 255) / 256)), dim3(256), 0, stream,
+                       cur_logp, ref_logp, old_logp, mask, ratio, kl, N);
+    if (hipGetLastError() != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, "ratio / kl launch failed");
+    return 0;
+}
+
+int rlk_ratio_kl_from_logp_bwd(const float* cur_logp, const float* ref_logp, const float* old_logp,
+                               const uint8_t* mask, const float* grad_ratio, const float* grad_kl,
+                               int64_t N, float* d_cur, hipStream_t stream)
+{
+    if (!cur_logp || !ref_logp || !old_logp || !d_cur) return rlk_fail(RLK_ERR_ARG, "null pointer");
+    if (N < 0) return rlk_fail(RLK_ERR_ARG, "bad sizes");
+    if (N == 0) return 0;
+    hipLaunchKernelGGL(ratio_kl_bwd_kernel, dim3(static_cast<unsigned>((N + 255) / 256)), dim3(256), 0, stream,
+                       cur_logp, ref_logp, old_logp, mask, grad_ratio, grad_kl, d_cur, N);
+    if (hipGetLastError() != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, "ratio / kl backward launch failed");
     return 0;
 }
 

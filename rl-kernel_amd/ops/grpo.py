@@ -161,6 +161,44 @@ class RocmGRPOFromLogpOp:
     group_advantages = staticmethod(group_advantages)
 
 
+class _RatioKLFromLogpFunction(torch.autograd.Function):
+    """``(ratio, kl)`` per token from current / reference / old log-probs, one launch each way;
+    differentiable w.r.t. the current log-probs only."""
+
+    @staticmethod
+    def forward(ctx, cur, ref, old, mask):
+        shape = cur.shape
+        dev = cur.device
+        cur_f, ref_f, old_f = (_f32(t).reshape(-1) for t in (cur, ref, old))
+        mask_u8 = mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8).reshape(-1)
+        n = cur_f.numel()
+        ratio = torch.empty(n, device=dev, dtype=torch.float32)
+        kl = torch.empty(n, device=dev, dtype=torch.float32)
+        with torch.cuda.device(dev):
+            rc = _native.load().rlk_ratio_kl_from_logp(
+                cur_f.data_ptr(), ref_f.data_ptr(), old_f.data_ptr(), mask_u8.data_ptr(), n,
+                ratio.data_ptr(), kl.data_ptr(), _stream(dev))
+        _native.check(rc, "rlk_ratio_kl_from_logp")
+        ctx.save_for_backward(cur_f, ref_f, old_f, mask_u8)
+        ctx.shape = shape
+        return ratio.view(shape), kl.view(shape)
+
+    @staticmethod
+    def backward(ctx, g_ratio, g_kl):
+        cur_f, ref_f, old_f, mask_u8 = ctx.saved_tensors
+        n = cur_f.numel()
+        gr = None if g_ratio is None else _f32(g_ratio).reshape(-1)
+        gk = None if g_kl is None else _f32(g_kl).reshape(-1)
+        d_cur = torch.empty(n, device=cur_f.device, dtype=torch.float32)
+        p = lambda t: None if t is None else t.data_ptr()
+        with torch.cuda.device(cur_f.device):
+            rc = _native.load().rlk_ratio_kl_from_logp_bwd(
+                cur_f.data_ptr(), ref_f.data_ptr(), old_f.data_ptr(), mask_u8.data_ptr(), p(gr), p(gk),
+                n, d_cur.data_ptr(), _stream(cur_f.device))
+        _native.check(rc, "rlk_ratio_kl_from_logp_bwd")
+        return d_cur.view(ctx.shape), None, None, None
+
+
 class RocmRatioKLOp:
     """Logits-fed ratio + k3 KL: mask-before-exp, so inactive positions give ratio 1 and kl 0
     (rl_engine/kernels/ops/pytorch/loss/ratio_kl.py:32-58 of the reference)."""
@@ -183,9 +221,7 @@ class RocmRatioKLOp:
         # both logit tensors in one scan launch (the reference's program reads both rows too:
         # rl_engine/kernels/ops/triton/loss/ratio_kl.py:46-60)
         logp_policy, logp_ref = differentiable_logp_pair_fp32(policy_logits, ref_logits, safe_ids)
-        delta = (logp_policy - old_logps.float()).masked_fill(~mask, 0.0)
-        diff = (logp_ref - logp_policy).masked_fill(~mask, 0.0)
-        return torch.exp(delta), torch.exp(diff) - diff - 1.0
+        return _RatioKLFromLogpFunction.apply(logp_policy, logp_ref, old_logps, mask)
 
 
 class RocmGRPOLossOp:

@@ -292,3 +292,48 @@ def test_epilogue_folded_into_the_forward_equals_the_two_step_route(dev, ops, b,
     (loss2 + 0.5 * kl2).backward()
     assert torch.equal(loss, loss2) and torch.equal(pol, pol2) and torch.equal(kl, kl2)
     assert torch.equal(hd.grad, hd2.grad) and torch.equal(wd.grad, wd2.grad)
+
+
+def test_ratio_kl_entry_points_match_the_closed_forms(dev):
+    """rlk_ratio_kl_from_logp / _bwd through the C ABI: values and the coefficient of the logits
+    gradient against the formulas of the reference's kernels (ratio = exp(cur - old),
+    kl = exp(d) - d - 1 with d = ref - cur, d/dcur = g_r * ratio + g_k * (1 - exp(d))), with and
+    without a mask and with either upstream gradient absent."""
+    from rl_kernel_amd import _native
+
+    lib = _native.load()
+    g = torch.Generator().manual_seed(21)
+    n = 1000
+    cur = torch.randn(n, generator=g) * 0.3 - 4.0
+    ref = cur + torch.randn(n, generator=g) * 0.2
+    old = cur + torch.randn(n, generator=g) * 0.2
+    mask = torch.rand(n, generator=g) > 0.3
+    gr, gk = torch.randn(n, generator=g), torch.randn(n, generator=g)
+    st = torch.cuda.current_stream().cuda_stream
+    cd, rd, od, md, grd, gkd = (t.to(dev) for t in (cur, ref, old, mask.view(torch.uint8), gr, gk))
+    ratio = torch.empty(n, device=dev)
+    kl = torch.empty(n, device=dev)
+    dcur = torch.empty(n, device=dev)
+    for m_cpu, m_dev in ((mask, md), (torch.ones(n, dtype=torch.bool), None)):
+        mp = None if m_dev is None else m_dev.data_ptr()
+        assert lib.rlk_ratio_kl_from_logp(cd.data_ptr(), rd.data_ptr(), od.data_ptr(), mp, n,
+                                          ratio.data_ptr(), kl.data_ptr(), st) == 0
+        delta = (cur - old).masked_fill(~m_cpu, 0.0)
+        d = (ref - cur).masked_fill(~m_cpu, 0.0)
+        assert torch.allclose(ratio.cpu(), torch.exp(delta), rtol=1e-6, atol=1e-7)
+        # exp(d) - d - 1 cancels near d = 0: the error is a few ulps of 1.0, not of the result
+        assert torch.allclose(kl.cpu(), torch.exp(d) - d - 1.0, rtol=1e-5, atol=5e-7)
+        assert torch.all(ratio.cpu()[~m_cpu] == 1.0) and torch.all(kl.cpu()[~m_cpu] == 0.0)
+        for use_r, use_k in ((True, True), (True, False), (False, True)):
+            assert lib.rlk_ratio_kl_from_logp_bwd(
+                cd.data_ptr(), rd.data_ptr(), od.data_ptr(), mp, grd.data_ptr() if use_r else None,
+                gkd.data_ptr() if use_k else None, n, dcur.data_ptr(), st) == 0
+            want = torch.zeros(n)
+            if use_r:
+                want = want + gr * torch.exp(cur - old)
+            if use_k:
+                want = want + gk * (1.0 - torch.exp(ref - cur))
+            want = want.masked_fill(~m_cpu, 0.0)
+            assert torch.allclose(dcur.cpu(), want, rtol=1e-5, atol=1e-6)
+    assert lib.rlk_ratio_kl_from_logp(None, rd.data_ptr(), od.data_ptr(), None, n, ratio.data_ptr(),
+                                      kl.data_ptr(), st) < 0
