@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "316f5378a63c3415",
-    "measured_at_commit": "663f4c5",
+    "kernel_source_sha16": "5fae77626fc08d8d",
+    "measured_at_commit": "c7783f6",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 51559718893,
-        "linear_logp_dz_kernel": 1968313923,
-        "linear_logp_dh_kernel": 1848738332,
-        "linear_logp_dw_kernel": 2177399221,
+        "linear_logp_fwd_kernel": 51922171043,
+        "linear_logp_dz_kernel": 1964798395,
+        "linear_logp_dh_kernel": 1837763095,
+        "linear_logp_dw_kernel": 2183703317,
     },
 }
 
