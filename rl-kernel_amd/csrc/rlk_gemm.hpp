@@ -47,6 +47,12 @@ typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 #ifndef RLK_LW
 #define RLK_LW 2  // direct-to-LDS: slices over which the loads of one K step are spread
 #endif
+// The persistent dZ and dH kernels stall more on operand loads than the forward: for them all loads
+// of a K step go out in the first slice of the window, a full K step ahead of their barrier (the
+// forward loses up to 1.4 % with that window).
+#ifndef RLK_LW_BWD
+#define RLK_LW_BWD 1
+#endif
 #ifndef RLK_RD
 #define RLK_RD 8  // direct-to-LDS: fragment reads issued per 8 MFMA slots (8 = one per slot)
 #endif
@@ -271,7 +277,7 @@ __device__ inline void static_for(F&& f)
     }
 }
 
-template <class T, bool A_KMAJOR, bool B_KMAJOR, int BK>
+template <class T, bool A_KMAJOR, bool B_KMAJOR, int BK, int LWIN = RLK_LW>
 struct TileGemmDtl;
 
 // Workgroup tile contraction.  acc[i][j] (+)= A rows x B rows over k in [0, K).
@@ -523,7 +529,7 @@ struct DtlIO {
     }
 };
 
-template <class T, bool A_KMAJOR, bool B_KMAJOR, int BK>
+template <class T, bool A_KMAJOR, bool B_KMAJOR, int BK, int LWIN>
 struct TileGemmDtl {
     static constexpr int TM = kTM;
     static constexpr int TN = kTN;
@@ -534,7 +540,7 @@ struct TileGemmDtl {
     static constexpr int PB = IOB::kPasses;
     static constexpr int NL = PA + PB;                 // loads per wavefront per K step
     static constexpr int NM = TM * TN;                 // MFMAs per slice
-    static constexpr int LW = RLK_LW;                  // load window in slices
+    static constexpr int LW = LWIN;                    // load window in slices
     static_assert(LW >= 1 && LW <= KK - 1, "load window must end before the barrier slice");
     static constexpr int kStageBytes = IOA::kBytes + IOB::kBytes;
     static constexpr int kSmemBytes = 2 * kStageBytes;

@@ -14,6 +14,18 @@
 #include "rlk_grpo.hpp"
 #include "rlk_tile_epilogue.hpp"
 
+// Load window of the persistent backward kernels (see RLK_LW_BWD), measured one kernel at a time
+// at the Llama head: dZ 3.5 % and dH 1.3 % faster with the early window, dW 2 % slower.
+#ifndef RLK_LW_DZ
+#define RLK_LW_DZ RLK_LW_BWD
+#endif
+#ifndef RLK_LW_DH
+#define RLK_LW_DH RLK_LW_BWD
+#endif
+#ifndef RLK_LW_DW
+#define RLK_LW_DW RLK_LW
+#endif
+
 namespace rlk {
 
 
@@ -431,7 +443,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
 {
     static_assert(!(GENERAL && CHAIN), "the chained variant covers full tiles only");
     using Gemm = TileGemm<T, false, false, BK>;
-    using Dtl = TileGemmDtl<T, false, false, BK>;
+    using Dtl = TileGemmDtl<T, false, false, BK, RLK_LW_DZ>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int wave = threadIdx.x >> 6;
     TileWalk walk(a.tok_tiles * a.v_tiles, a.v_tiles, a.tok_tiles);
@@ -595,7 +607,7 @@ template <class T, int BK, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
 {
     using Gemm = TileGemm<T, true, false, BK>;
-    using Dtl = TileGemmDtl<T, true, false, BK>;
+    using Dtl = TileGemmDtl<T, true, false, BK, RLK_LW_DH>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     f32x16_t acc[kTM][kTN];
     if constexpr (CHAIN) {
@@ -780,7 +792,7 @@ template <class T, int BK, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
 {
     using Gemm = TileGemm<T, true, true, BK>;
-    using Dtl = TileGemmDtl<T, true, true, BK>;
+    using Dtl = TileGemmDtl<T, true, true, BK, RLK_LW_DW>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     TileWalk walk(a.v_tiles * a.h_tiles, a.v_tiles, a.h_tiles);
     if (!walk.valid()) return;
