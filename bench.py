@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "5fae77626fc08d8d",
-    "measured_at_commit": "c7783f6",
+    "kernel_source_sha16": "ed990790b256785d",
+    "measured_at_commit": "d67990c",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 51922171043,
-        "linear_logp_dz_kernel": 1964798395,
-        "linear_logp_dh_kernel": 1837763095,
-        "linear_logp_dw_kernel": 2183703317,
+        "linear_logp_fwd_kernel": 51472576218,
+        "linear_logp_dz_kernel": 1959997973,
+        "linear_logp_dh_kernel": 1935593557,
+        "linear_logp_dw_kernel": 2160175852,
     },
 }
 
