@@ -44,13 +44,13 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
     "kernel_source_sha16": "ed990790b256785d",
-    "measured_at_commit": "d67990c",
+    "measured_at_commit": "43286d2",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 51472576218,
-        "linear_logp_dz_kernel": 1959997973,
-        "linear_logp_dh_kernel": 1935593557,
-        "linear_logp_dw_kernel": 2160175852,
+        "linear_logp_fwd_kernel": 52009413181,
+        "linear_logp_dz_kernel": 1963094859,
+        "linear_logp_dh_kernel": 1893046182,
+        "linear_logp_dw_kernel": 2162991501,
     },
 }
 
