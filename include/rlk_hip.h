@@ -319,13 +319,6 @@ int rlk_ratio_kl_from_logp_bwd(const float* cur_logp, const float* ref_logp, con
 int rlk_group_advantages(const float* rewards, const int64_t* group_bounds, int64_t num_groups,
                          float eps, float* advantages, rlk_stream_t stream);
 
-/* ------------------------------------------------------------------------------------------ *
- * Hardware-contract self test (no counterpart in the reference): checks that the gfx950
- * transposing LDS read delivers the MFMA operand layout the backward contractions rely on.
- * out: device int32[512]; out[l*8 + e] must equal (8*(l/32) + e) * 256 + (l % 32).
- * ------------------------------------------------------------------------------------------ */
-int rlk_selftest_transpose_read(int32_t* out, rlk_stream_t stream);
-
 #ifdef __cplusplus
 }
 #endif

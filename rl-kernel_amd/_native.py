@@ -62,7 +62,6 @@ SIGNATURES = {
     "rlk_ratio_kl_from_logp": (_c.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp]),
     "rlk_ratio_kl_from_logp_bwd": (_c.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp]),
     "rlk_group_advantages": (_c.c_int, [_vp, _vp, _i64, _f32, _vp, _vp]),
-    "rlk_selftest_transpose_read": (_c.c_int, [_vp, _vp]),
 }
 
 _lib = None

@@ -14,17 +14,43 @@
 #include "rlk_grpo.hpp"
 #include "rlk_tile_epilogue.hpp"
 
-// Load window of the persistent backward kernels (see RLK_LW_BWD), measured one kernel at a time
-// at the Llama head: dZ 3.5 % and dH 1.3 % faster with the early window, dW 2 % slower.
-#ifndef RLK_LW_DZ
-#define RLK_LW_DZ RLK_LW_BWD
+// Load windows (MFMA slots of a K step's second slice over which its 8 loads are spread, see
+// TileGemmDtl), measured one kernel at a time at the Llama head: the persistent dZ and dH kernels
+// are faster with all loads out early, the forward and dW with the loads spread over the slice.
+#ifndef RLK_X_WIN_FWD
+#define RLK_X_WIN_FWD 32
 #endif
-#ifndef RLK_LW_DH
-#define RLK_LW_DH RLK_LW_BWD
+#ifndef RLK_X_WIN_DZ
+#define RLK_X_WIN_DZ 16
 #endif
-#ifndef RLK_LW_DW
-#define RLK_LW_DW RLK_LW
+#ifndef RLK_X_WIN_DH
+#define RLK_X_WIN_DH 16
 #endif
+#ifndef RLK_X_WIN_DW
+#define RLK_X_WIN_DW 32
+#endif
+#ifndef RLK_X_FWD_REFETCH
+#define RLK_X_FWD_REFETCH false
+#endif
+#ifndef RLK_X_DZ_YOUNGER
+#define RLK_X_DZ_YOUNGER 0
+#endif
+#ifndef RLK_X_SAMETILE
+#define RLK_X_SAMETILE 1  // experiment: 0 = every workgroup fetches tile 0 (all loads hit L2)
+#endif
+#ifndef RLK_X_DH_YOUNGER
+#define RLK_X_DH_YOUNGER (Acc16::TM * Acc16::TN / 2)
+#endif
+#ifndef RLK_X_DW_YOUNGER
+#define RLK_X_DW_YOUNGER (Acc16::TM * Acc16::TN / 2)
+#endif
+constexpr int kWinFwd = RLK_X_WIN_FWD;
+constexpr int kWinDz = RLK_X_WIN_DZ;
+constexpr int kWinDh = RLK_X_WIN_DH;
+constexpr int kWinDw = RLK_X_WIN_DW;
+// The forward carries the first fragments of the next tile through the softmax update (false) or
+// reads them again from LDS afterwards (true).
+constexpr bool kFwdRefetch = RLK_X_FWD_REFETCH;
 
 namespace rlk {
 
@@ -67,8 +93,10 @@ struct FwdArgs {
 template <class T, int BK, bool GENERAL>
 __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
 {
-    constexpr int TM = kTM, TN = kTN;
+    using AT = Acc16;
+    constexpr int TM = AT::TM, TN = AT::TN;
     using Gemm = TileGemm<T, false, false, BK>;
+    using Dtl = TileGemmDtl<T, false, false, BK, kWinFwd>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     int tb, sp;
@@ -88,7 +116,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
     int tgt[TN];  // target id relative to the shard, -1 when not in [0, V)
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int t = wn * (TN * 32) + j * 32 + (lane & 31);
+        const int t = wn * (TN * 16) + AT::col(j, lane);
         int64_t g = a.targets[tok0 + (t < tok_valid ? t : tok_valid - 1)] - a.vocab_start;
         tgt[j] = (g >= 0 && g < a.V) ? static_cast<int>(g) : -1;
     }
@@ -101,30 +129,37 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
         }
     };
 
-    // Merge of one head's state: the two half-wave row groups (same token, different vocab rows),
-    // then the wavefronts along M through LDS, in a fixed order; written to that head's partial
-    // arrays.  The LDS patch lies behind the pipeline stages, so the merge of the first head can run
-    // while the second head's first K steps are already on their way.
-    float* red = reinterpret_cast<float*>(smem + TileGemmDtl<T, false, false, BK>::kSmemBytes);  // [kWM][256 tokens][3]
-    static_assert(TileGemmDtl<T, false, false, BK>::kSmemBytes + kWM * 256 * 3 * 4 <= Gemm::kSmemBytes,
-                  "merge patch must fit the kernel's LDS");
+    // Merge of one head's state: the four lane groups of a wavefront (same token, different vocab
+    // rows; groups 16 apart first, then 32 apart), then the wavefronts along M through LDS, in a
+    // fixed order; written to that head's partial arrays.  The LDS patch lies behind the pipeline
+    // stages, so the merge of the first head can run while the second head's first K steps are
+    // already on their way.
+    float* red = reinterpret_cast<float*>(smem + Dtl::kSmemBytes);  // [kWM][256 tokens][3]
+    static_assert(Dtl::kSmemBytes + kWM * 256 * 3 * 4 <= Gemm::kSmemBytes, "merge patch must fit the kernel's LDS");
     auto flush_state = [&](float* pm, float* ps, float* pz) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const float m2 = __shfl_xor(m[j], 32);
-            const float s2 = __shfl_xor(s[j], 32);
-            const float z2 = __shfl_xor(zt[j], 32);
-            const float mm = fmaxf(m[j], m2);
-            const float mref = mm == -INFINITY ? 0.f : mm;
-            const float lo_m = lane < 32 ? m[j] : m2, hi_m = lane < 32 ? m2 : m[j];
-            const float lo_s = lane < 32 ? s[j] : s2, hi_s = lane < 32 ? s2 : s[j];
-            const float ss = lo_s * __builtin_amdgcn_exp2f(lo_m - mref) +
-                             hi_s * __builtin_amdgcn_exp2f(hi_m - mref);
-            if (lane < 32) {
-                float* dst = red + ((wm * 256) + wn * (TN * 32) + j * 32 + lane) * 3;
-                dst[0] = mm;
-                dst[1] = ss;
-                dst[2] = zt[j] + z2;
+            float mj = m[j], sj = s[j], zj = zt[j];
+#pragma unroll
+            for (int off = 16; off <= 32; off <<= 1) {
+                const float m2 = __shfl_xor(mj, off);
+                const float s2 = __shfl_xor(sj, off);
+                const float z2 = __shfl_xor(zj, off);
+                const float mm = fmaxf(mj, m2);
+                const float mref = mm == -INFINITY ? 0.f : mm;
+                // both partners evaluate the same expression: the lower group's term first
+                const bool low = (lane & off) == 0;
+                const float lo_m = low ? mj : m2, hi_m = low ? m2 : mj;
+                const float lo_s = low ? sj : s2, hi_s = low ? s2 : sj;
+                sj = lo_s * __builtin_amdgcn_exp2f(lo_m - mref) + hi_s * __builtin_amdgcn_exp2f(hi_m - mref);
+                mj = mm;
+                zj = (low ? zj : z2) + (low ? z2 : zj);
+            }
+            if (lane < 16) {
+                float* dst = red + ((wm * 256) + wn * (TN * 16) + j * 16 + lane) * 3;
+                dst[0] = mj;
+                dst[1] = sj;
+                dst[2] = zj;
             }
         }
         __syncthreads();
@@ -154,31 +189,25 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
     auto tile_origin = [&](int head, int vt) {
         return (head == 0 ? a.weight : a.weight2) + static_cast<int64_t>(vt) * 256 * a.H;
     };
-    if (!GENERAL && RLK_DTL != 0 && RLK_STREAM != 0 && a.H % BK == 0 && a.H >= 2 * BK && t0 < t1) {
+    if (!GENERAL && a.H % BK == 0 && a.H >= 2 * BK && t0 < t1) {
         // every tile is full: one pipeline runs through all tiles of the range (and then through
         // the same range of the second head), the K loop of a tile already fetching the head of the
         // next one while the softmax update runs (the pipeline looks two K steps ahead, which stays
         // within the next tile from two steps up)
-        using Dtl = TileGemmDtl<T, false, false, BK>;
         typename Dtl::Stream st;
         Dtl::begin(st, Operand{tile_origin(0, t0), a.H, 256}, B, a.H, smem);
         for (int head = 0; head < n_heads; ++head) {
             reset_state();
             for (int vt = t0; vt < t1; ++vt) {
-                f32x16_t acc[TM][TN];
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+                f32x4_t acc[TM][TN];
+                zero_acc(acc);
                 const void* next = vt + 1 < t1 ? tile_origin(head, vt + 1)
                                                : (head + 1 < n_heads ? tile_origin(head + 1, t0)
                                                                      : tile_origin(head, vt));
-                Dtl::tile(st, next, B.base, acc, smem);
+                Dtl::template tile<kFwdRefetch>(st, next, B.base, acc, smem);
                 const float* bias = head == 0 ? a.bias : a.bias2;
-                if (bias != nullptr) add_bias(acc, bias, vt * 256 + wm * (TM * 32), lane);  // uniform
-                fwd_epilogue<GENERAL>(acc, a, nullptr, vt * 256 + wm * (TM * 32), lane, tgt, m, s, zt);
+                if (bias != nullptr) add_bias<AT>(acc, bias, vt * 256 + wm * (TM * 16), lane);  // uniform
+                fwd_epilogue<GENERAL, AT>(acc, a, nullptr, vt * 256 + wm * (TM * 16), lane, tgt, m, s, zt);
             }
             if (head == 0)
                 flush_state(a.part_m, a.part_s, a.part_z);
@@ -193,16 +222,11 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
             for (int vt = t0; vt < t1; ++vt) {
                 const int v0 = vt * 256;
                 Operand A{tile_origin(head, vt), a.H, min(256, a.V - v0)};
-                f32x16_t acc[TM][TN];
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+                f32x4_t acc[TM][TN];
+                zero_acc(acc);
                 Gemm::run(A, B, a.H, acc, smem);
-                if (!GENERAL && bias != nullptr) add_bias(acc, bias, v0 + wm * (TM * 32), lane);  // uniform
-                fwd_epilogue<GENERAL>(acc, a, bias, v0 + wm * (TM * 32), lane, tgt, m, s, zt);
+                if (!GENERAL && bias != nullptr) add_bias<AT>(acc, bias, v0 + wm * (TM * 16), lane);  // uniform
+                fwd_epilogue<GENERAL, AT>(acc, a, bias, v0 + wm * (TM * 16), lane, tgt, m, s, zt);
             }
             if (head == 0)
                 flush_state(a.part_m, a.part_s, a.part_z);
@@ -336,99 +360,102 @@ struct DzArgs {
 // LDS each wavefront needs to turn its part of a dZ tile into full rows: 64 tokens x 32 vocab
 // columns of 16-bit values, 64 bytes per token row, no padding.
 constexpr int kDzStageBytes = 64 * 64;
-// Global stores one wavefront issues per dZ tile (kTM groups x 8 row batches), all unconditional.
-constexpr int kDzStores = kTM * 8;
+// Global stores one wavefront issues per dZ tile (four 32-row groups x 8 row batches), all unconditional.
+constexpr int kDzStores = (Acc16::TM / 2) * 8;
 
 // dZ epilogue of one 256 x 256 tile.  A wavefront owns 128 vocab rows x 64 tokens of the tile; for
-// each of its four 32-row groups it writes the rounded values into its private LDS patch as
-// [token][vocab] rows and reads them back row-wise, so that the tile leaves in runs of 64
-// contiguous bytes per token.  Only the wavefront itself touches its patch: no workgroup barrier.
-// The 8-byte units of a row are XOR-swizzled with (token / 4) & 7, which makes both the writes
-// (32 tokens, same unit) and the reads (4 rows x 8 units) conflict-free.
+// each of its four 32-row groups (two 16-row MFMA tiles) it writes the rounded values into its
+// private LDS patch as [token][vocab] rows and reads them back row-wise, so that the tile leaves
+// in runs of 64 contiguous bytes per token.  Only the wavefront itself touches its patch: no
+// workgroup barrier.  The 8-byte units of a row are XOR-swizzled with 2 * ((token / 4) & 3), which
+// makes both the writes (16 tokens x 2 lane groups per pass) and the reads (4 rows x 8 units)
+// conflict-free.
 template <class T, bool GENERAL>
-__device__ inline void dz_epilogue(const f32x16_t (&acc)[kTM][kTN], const DzArgs& a, int vt, int tt,
+__device__ inline void dz_epilogue(const f32x4_t (&acc)[Acc16::TM][Acc16::TN], const DzArgs& a, int vt, int tt,
                                    char* stage)
 {
-    constexpr int TM = kTM, TN = kTN;
+    using AT = Acc16;
+    constexpr int TM = AT::TM, TN = AT::TN;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
     const int tok0 = tt * 256, v0 = vt * 256;
     const int tok_rows = min(256, a.tok_valid - tok0);
     const float gscale = a.scales[0];
-    const int vw = v0 + wm * (TM * 32);
-    const int hi = lane >> 5;
+    const int vw = v0 + wm * (TM * 16);
+    const int grp = lane >> 4;  // this lane holds rows 4 * grp + 0..3 of every 16-row tile
 
     float gs[TN], nlse2[TN];
-    int etgt[TN];  // register index (i*16 + r) of the target row in this lane, or -1
+    int etgt[TN];  // register index (i*4 + r) of the target row in this lane, or -1
     bool any_target = false;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int tl = wn * (TN * 32) + j * 32 + (lane & 31);
+        const int tl = wn * (TN * 16) + AT::col(j, lane);
         const int tc = tok0 + (tl < tok_rows ? tl : tok_rows - 1);
         const int64_t tg = a.targets[tc];
         const bool live = tl < tok_rows && !(a.use_ignore && tg == a.ignore_index);
         gs[j] = live ? a.grad[tc] * gscale : 0.f;
         nlse2[j] = -a.lse[tc] * kLog2e;
         const int64_t trel = tg - a.v_global0 - vw;
-        const int tr = (trel >= 0 && trel < TM * 32) ? static_cast<int>(trel) : -1;
-        const int x = tr & 31;
-        etgt[j] = (tr >= 0 && ((x >> 2) & 1) == hi) ? ((tr >> 5) * 16 + (x >> 3) * 4 + (x & 3)) : -1;
+        etgt[j] = (trel >= 0 && trel < TM * 16) ? AT::reg_of_row(static_cast<int>(trel), lane) : -1;
         any_target = any_target || etgt[j] >= 0;
     }
     // the one-hot term is added only when some lane of the wavefront owns its target row here
     const bool hot = __builtin_amdgcn_ballot_w64(any_target) != 0;  // uniform
 
-    uint16_t* dtile = a.dz + static_cast<int64_t>(tok0 + wn * (TN * 32)) * a.ldz + vw;
-    auto stage_rows = [&](auto ic, auto hot_c) {
-        constexpr int i = decltype(ic)::value;
+    uint16_t* dtile = a.dz + static_cast<int64_t>(tok0 + wn * (TN * 16)) * a.ldz + vw;
+    auto stage_rows = [&](auto ipc, auto hot_c) {
+        constexpr int ip = decltype(ipc)::value;  // 32-row group = MFMA tiles 2 ip and 2 ip + 1
         constexpr bool HOT = decltype(hot_c)::value;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int t = j * 32 + (lane & 31);  // token row inside the wavefront's patch
+            const int t = j * 16 + (lane & 15);  // token row inside the wavefront's patch
             char* srow = stage + t * 64;
-            const int sw = (t >> 2) & 7;
-            auto prob = [&](int r) -> float {
-                float z = acc[i][j][r];
-                if (GENERAL) {
-                    const int v = vw + i * 32 + acc_row(r, lane);
-                    if (a.bias != nullptr) z += a.bias[v < a.v_valid ? v : a.v_valid - 1];
-                    return v < a.v_valid ? __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2[j])) : 0.f;
-                }
-                return __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2[j]));
-            };
+            const int sw = ((t >> 2) & 3) << 1;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
+            for (int ii = 0; ii < 2; ++ii) {
+                constexpr int i0 = 2 * ip;
+                const int i = i0 + ii;
                 float d[4];
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    if constexpr (HOT) {
-                        const float hit = (etgt[j] == i * 16 + q * 4 + c) ? gs[j] : 0.f;
-                        d[c] = fmaf(-gs[j], prob(q * 4 + c), hit);
+                    float z = acc[i][j][c];
+                    float pr;
+                    if (GENERAL) {
+                        const int v = vw + i * 16 + 4 * grp + c;
+                        if (a.bias != nullptr) z += a.bias[v < a.v_valid ? v : a.v_valid - 1];
+                        pr = v < a.v_valid ? __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2[j])) : 0.f;
                     } else {
-                        d[c] = -gs[j] * prob(q * 4 + c);
+                        pr = __builtin_amdgcn_exp2f(fmaf(z, a.scale2, nlse2[j]));
+                    }
+                    if constexpr (HOT) {
+                        const float hit = (etgt[j] == i * 4 + c) ? gs[j] : 0.f;
+                        d[c] = fmaf(-gs[j], pr, hit);
+                    } else {
+                        d[c] = -gs[j] * pr;
                     }
                 }
-                // rows 8q + 4hi + 0..3 of this 32-row group: unit 2q + hi of the token's row
-                *reinterpret_cast<u32x2_t*>(srow + (((2 * q + hi) ^ sw) * 8)) =
+                // rows 16 ii + 4 grp + 0..3 of this 32-row group: unit 4 ii + grp of the token's row
+                *reinterpret_cast<u32x2_t*>(srow + (((4 * ii + grp) ^ sw) * 8)) =
                     u32x2_t{T::pack2(d[0], d[1]), T::pack2(d[2], d[3])};
             }
         }
     };
-    static_for<0, TM>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
+    static_for<0, TM / 2>([&](auto ipc) {
+        constexpr int ip = decltype(ipc)::value;
         if (hot)
-            stage_rows(ic, std::true_type{});
+            stage_rows(ipc, std::true_type{});
         else
-            stage_rows(ic, std::false_type{});
+            stage_rows(ipc, std::false_type{});
         __builtin_amdgcn_wave_barrier();
         // copy-out: 8 lanes move one token row (64 bytes), 8 rows per instruction
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
             const int row = it * 8 + (lane >> 3);
             const int u = lane & 7;
-            const u32x2_t v = *reinterpret_cast<const u32x2_t*>(stage + row * 64 + ((u ^ ((row >> 2) & 7)) * 8));
-            *reinterpret_cast<u32x2_t*>(dtile + static_cast<int64_t>(row) * a.ldz + i * 32 + u * 4) = v;
+            const u32x2_t v =
+                *reinterpret_cast<const u32x2_t*>(stage + row * 64 + ((u ^ (((row >> 2) & 3) << 1)) * 8));
+            *reinterpret_cast<u32x2_t*>(dtile + static_cast<int64_t>(row) * a.ldz + ip * 32 + u * 4) = v;
         }
         __builtin_amdgcn_wave_barrier();
     });
@@ -442,17 +469,18 @@ template <class T, int BK, bool GENERAL, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
 {
     static_assert(!(GENERAL && CHAIN), "the chained variant covers full tiles only");
+    using AT = Acc16;
     using Gemm = TileGemm<T, false, false, BK>;
-    using Dtl = TileGemmDtl<T, false, false, BK, RLK_LW_DZ>;
+    using Dtl = TileGemmDtl<T, false, false, BK, kWinDz>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int wave = threadIdx.x >> 6;
     TileWalk walk(a.tok_tiles * a.v_tiles, a.v_tiles, a.tok_tiles);
     if (!walk.valid()) return;
     int vt, tt;
     walk.coords(false, vt, tt);
-    auto w_origin = [&](int v) { return a.weight + static_cast<int64_t>(v + a.v_tile_lo) * 256 * a.H; };
-    auto h_origin = [&](int t) { return a.hidden + static_cast<int64_t>(t) * 256 * a.H; };
-    f32x16_t acc[kTM][kTN];
+    auto w_origin = [&](int v) { return a.weight + static_cast<int64_t>(v + a.v_tile_lo) * RLK_X_SAMETILE * 256 * a.H; };
+    auto h_origin = [&](int t) { return a.hidden + static_cast<int64_t>(t) * RLK_X_SAMETILE * 256 * a.H; };
+    f32x4_t acc[AT::TM][AT::TN];
     if constexpr (CHAIN) {
         char* stage = smem + Dtl::kSmemBytes + wave * kDzStageBytes;
         typename Dtl::Stream st;
@@ -462,10 +490,9 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
             int nvt = vt, ntt = tt;
             if (more) walk.coords(true, nvt, ntt);
             zero_acc(acc);
-            Dtl::template tile<true, kDzStores / 2>(st, w_origin(nvt), h_origin(ntt), acc, smem, true);
-            if (more) Dtl::fetch_ahead(st, smem);
+            Dtl::template tile<true, RLK_X_DZ_YOUNGER>(st, w_origin(nvt), h_origin(ntt), acc, smem, true);
             if (a.bias != nullptr)  // uniform
-                add_bias(acc, a.bias, (vt + a.v_tile_lo) * 256 + (wave / kWN) * (kTM * 32), threadIdx.x & 63);
+                add_bias<AT>(acc, a.bias, (vt + a.v_tile_lo) * 256 + (wave / kWN) * (AT::TM * 16), threadIdx.x & 63);
             dz_epilogue<T, GENERAL>(acc, a, vt + a.v_tile_lo, tt, stage);
             if (!more) break;
             walk.advance();
@@ -482,7 +509,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
             zero_acc(acc);
             Gemm::run(A, B, a.H, acc, smem);  // ends with a barrier: LDS is free
             if (!GENERAL && a.bias != nullptr)  // uniform
-                add_bias(acc, a.bias, v0 + (wave / kWN) * (kTM * 32), threadIdx.x & 63);
+                add_bias<AT>(acc, a.bias, v0 + (wave / kWN) * (AT::TM * 16), threadIdx.x & 63);
             dz_epilogue<T, GENERAL>(acc, a, vt + a.v_tile_lo, tt, smem + wave * kDzStageBytes);
             if (!walk.has_next()) break;
             walk.advance();
@@ -515,82 +542,87 @@ struct DhArgs {
 };
 
 // Epilogue of one dH tile.  The read-modify-write of the running fp32 partial is latency-bound, so
-// it runs in two batches (one per 32-token column group): the 16 reads of a batch are all issued
-// before the first use, then added and stored.  FULL (the tile lies inside the chunk and inside
-// H): addresses are a uniform tile origin plus a 32-bit lane offset and no predicates are needed;
-// otherwise rows and columns are clamped for the reads and predicated for the stores.
+// it runs in two batches (one per pair of 16-token column groups): the 16 reads of a batch are all
+// issued before the first use, then added and stored.  FULL (the tile lies inside the chunk and
+// inside H): addresses are a uniform tile origin plus a 32-bit lane offset and no predicates are
+// needed; otherwise rows and columns are clamped for the reads and predicated for the stores.
 // The tile covers hidden columns [h0, h0 + 256) and owns those from h_min on (h_min > h0 for the
 // last tile of a persistent walk when H is not a multiple of 256: it is shifted back to end at H
 // and must leave the columns of its left neighbour alone).
 template <class T, bool FULL>
-__device__ inline void dh_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const DhArgs& a, int tt,
+__device__ inline void dh_epilogue_impl(const f32x4_t (&acc)[Acc16::TM][Acc16::TN], const DhArgs& a, int tt,
                                         int h0, int h_min, float* acc_dst, bool first, bool last)
 {
-    constexpr int TM = kTM, TN = kTN;
+    using AT = Acc16;
+    constexpr int TM = AT::TM, TN = AT::TN;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
     const int tok0 = tt * 256;
     const float oscale = a.scales[1];
-    const int hbase = h0 + wm * (TM * 32) + 4 * (lane >> 5);  // + i * 32 + 8 * q
+    const int hbase = h0 + wm * (TM * 16) + 4 * (lane >> 4);  // + i * 16
     const uint32_t ldh = static_cast<uint32_t>(a.H);
     // FULL: byte offsets inside the tile stay below 256 * H * 4 (32 bits)
     const int64_t origin = static_cast<int64_t>(tok0) * a.H + h0;
     char* acc_tile = reinterpret_cast<char*>(acc_dst + origin);
     char* out_tile = reinterpret_cast<char*>(a.out + origin);
-    const uint32_t lane_el = static_cast<uint32_t>(wn * (TN * 32) + (lane & 31)) * ldh +
-                             static_cast<uint32_t>(wm * (TM * 32) + 4 * (lane >> 5));
+    const uint32_t lane_el = static_cast<uint32_t>(wn * (TN * 16) + (lane & 15)) * ldh +
+                             static_cast<uint32_t>(wm * (TM * 16) + 4 * (lane >> 4));
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int tl = tok0 + wn * (TN * 32) + j * 32 + (lane & 31);
-        const bool tok_ok = FULL || tl < a.tok_valid;
-        const int64_t trow = static_cast<int64_t>(tok_ok ? tl : a.tok_valid - 1) * a.H;
-        f32x4_t old[TM][4];
+    for (int jb = 0; jb < TN; jb += 2) {
+        f32x4_t old[2][TM];
+        bool tok_ok[2];
+        int64_t trow[2];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = jb + jj;
+            const int tl = tok0 + wn * (TN * 16) + AT::col(j, lane);
+            tok_ok[jj] = FULL || tl < a.tok_valid;
+            trow[jj] = static_cast<int64_t>(tok_ok[jj] ? tl : a.tok_valid - 1) * a.H;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                old[i][q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < TM; ++i) {
+                old[jj][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
                 if (!first) {  // uniform
                     if (FULL) {
-                        const char* rowp = acc_tile + (static_cast<size_t>(j * 32) * ldh + (i * 32 + 8 * q)) * 4u;
-                        old[i][q] = *reinterpret_cast<const f32x4_t*>(rowp + lane_el * 4u);
+                        const char* rowp = acc_tile + (static_cast<size_t>(j * 16) * ldh + i * 16) * 4u;
+                        old[jj][i] = *reinterpret_cast<const f32x4_t*>(rowp + lane_el * 4u);
                     } else {
-                        const int h = hbase + i * 32 + 8 * q;
-                        old[i][q] = *reinterpret_cast<const f32x4_t*>(acc_dst + trow + (h < a.H ? h : 0));
+                        const int h = hbase + i * 16;
+                        old[jj][i] = *reinterpret_cast<const f32x4_t*>(acc_dst + trow[jj] + (h < a.H ? h : 0));
                     }
                 }
             }
+        }
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = jb + jj;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int h = hbase + i * 32 + 8 * q;
-                f32x4_t v{acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
-                          acc[i][j][q * 4 + 3]};
-                v += old[i][q];
-                const size_t uni = static_cast<size_t>(j * 32) * ldh + (i * 32 + 8 * q);  // uniform
-                if (FULL || (tok_ok && h >= h_min && h < a.H)) {  // H % 8 == 0: a quad is all-in or all-out
+            for (int i = 0; i < TM; ++i) {
+                const int h = hbase + i * 16;
+                const f32x4_t v = acc[i][j] + old[jj][i];
+                const size_t uni = static_cast<size_t>(j * 16) * ldh + i * 16;  // uniform
+                if (FULL || (tok_ok[jj] && h >= h_min && h < a.H)) {  // H % 8 == 0: a quad is all-in or all-out
                     if (last) {
                         u32x2_t pk{T::pack2(v.x * oscale, v.y * oscale), T::pack2(v.z * oscale, v.w * oscale)};
                         if (FULL)
                             *reinterpret_cast<u32x2_t*>(out_tile + uni * 2u + lane_el * 2u) = pk;
                         else
-                            *reinterpret_cast<u32x2_t*>(a.out + trow + h) = pk;
+                            *reinterpret_cast<u32x2_t*>(a.out + trow[jj] + h) = pk;
                     } else {
                         if (FULL)
                             *reinterpret_cast<f32x4_t*>(acc_tile + uni * 4u + lane_el * 4u) = v;
                         else
-                            *reinterpret_cast<f32x4_t*>(acc_dst + trow + h) = v;
+                            *reinterpret_cast<f32x4_t*>(acc_dst + trow[jj] + h) = v;
                     }
                 }
             }
+        }
     }
 }
 
 // Returns whether the tile was full (then every wavefront issued all its stores unconditionally).
 template <class T>
-__device__ inline bool dh_epilogue(const f32x16_t (&acc)[kTM][kTN], const DhArgs& a, int tt, int h0,
+__device__ inline bool dh_epilogue(const f32x4_t (&acc)[Acc16::TM][Acc16::TN], const DhArgs& a, int tt, int h0,
                                    int h_min, float* acc_dst, bool first, bool last)
 {
     const bool full = tt * 256 + 256 <= a.tok_valid && h0 + 256 <= a.H && h_min == h0;  // uniform
@@ -607,9 +639,9 @@ template <class T, int BK, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
 {
     using Gemm = TileGemm<T, true, false, BK>;
-    using Dtl = TileGemmDtl<T, true, false, BK, RLK_LW_DH>;
+    using Dtl = TileGemmDtl<T, true, false, BK, kWinDh>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    f32x16_t acc[kTM][kTN];
+    f32x4_t acc[Acc16::TM][Acc16::TN];
     if constexpr (CHAIN) {
         TileWalk walk(a.tok_tiles * a.h_tiles, a.tok_tiles, a.h_tiles);
         if (!walk.valid()) return;
@@ -617,8 +649,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
         walk.coords(false, tt, ht);
         // first hidden column of h tile `h`: the last tile is shifted back so that it ends at H
         auto h_col = [&](int h) { return min(h * 256, a.H - 256); };
-        auto w_origin = [&](int h) { return a.weight + h_col(h); };
-        auto z_origin = [&](int t) { return a.dz + static_cast<int64_t>(t) * 256 * a.ldz; };
+        auto w_origin = [&](int h) { return a.weight + h_col(h) * RLK_X_SAMETILE; };
+        auto z_origin = [&](int t) { return a.dz + static_cast<int64_t>(t) * RLK_X_SAMETILE * 256 * a.ldz; };
         typename Dtl::Stream st;
         bool counted = false;
         Dtl::begin(st, Operand{w_origin(ht), a.H, 256}, Operand{z_origin(tt), a.ldz, 256}, a.v_valid, smem);
@@ -627,9 +659,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
             int ntt = tt, nht = ht;
             if (more) walk.coords(true, ntt, nht);
             zero_acc(acc);
-            // a full tile's epilogue issues kTM * kTN * 4 unconditional stores per wavefront
-            Dtl::template tile<true, kTM * kTN * 2>(st, w_origin(nht), z_origin(ntt), acc, smem, counted);
-            if (more) Dtl::fetch_ahead(st, smem);
+            // a full tile's epilogue issues TM * TN unconditional stores per wavefront
+            Dtl::template tile<true, RLK_X_DH_YOUNGER>(st, w_origin(nht), z_origin(ntt), acc, smem, counted);
             counted = dh_epilogue<T>(acc, a, tt, h_col(ht), ht * 256, a.acc, a.first != 0, a.last != 0);
             if (!more) break;
             walk.advance();
@@ -714,68 +745,74 @@ struct DwArgs {
 
 // Epilogue of one dW tile.  Orientation: M (accumulator registers) = hidden column, N (lane) =
 // vocab row, so a lane holds 4 consecutive columns of one dW row and the read-modify-write of the
-// fp32 tile moves 16 bytes per lane.  It is latency-bound and therefore runs in two batches (one
-// per 32-row group): the 16 reads of a batch are issued before the first use.  FULL (the tile lies
-// inside the piece and inside H): a uniform tile origin plus a 32-bit lane offset, no predicates;
-// otherwise clamped reads and predicated stores.
+// fp32 tile moves 16 bytes per lane (the four lane groups of a 16 x 16 tile make 64 contiguous
+// bytes per row).  It is latency-bound and therefore runs in two batches (one per pair of 16-row
+// groups): the 16 reads of a batch are issued before the first use.  FULL (the tile lies inside the
+// piece and inside H): a uniform tile origin plus a 32-bit lane offset, no predicates; otherwise
+// clamped reads and predicated stores.
 // The tile covers hidden columns [h0, h0 + 256) and owns those from h_min on (see dh_epilogue_impl).
 template <bool FULL>
-__device__ inline void dw_epilogue_impl(const f32x16_t (&acc)[kTM][kTN], const DwArgs& a, int vt, int h0,
-                                        int h_min)
+__device__ inline void dw_epilogue_impl(const f32x4_t (&acc)[Acc16::TM][Acc16::TN], const DwArgs& a, int vt,
+                                        int h0, int h_min)
 {
-    constexpr int TM = kTM, TN = kTN;
+    using AT = Acc16;
+    constexpr int TM = AT::TM, TN = AT::TN;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave / kWN, wn = wave % kWN;
     const int v0 = vt * 256;
     const float oscale = a.scales[1];
-    const int hbase = h0 + wm * (TM * 32) + 4 * (lane >> 5);  // + i * 32 + 8 * q
+    const int hbase = h0 + wm * (TM * 16) + 4 * (lane >> 4);  // + i * 16
     const uint32_t ldw = static_cast<uint32_t>(a.H);
     // FULL: byte offsets inside the tile stay below 256 * H * 4 (32 bits)
     char* tile = reinterpret_cast<char*>(a.dw + static_cast<int64_t>(v0) * a.H + h0);
-    const uint32_t lane_el = static_cast<uint32_t>(wn * (TN * 32) + (lane & 31)) * ldw +
-                             static_cast<uint32_t>(wm * (TM * 32) + 4 * (lane >> 5));
+    const uint32_t lane_el = static_cast<uint32_t>(wn * (TN * 16) + (lane & 15)) * ldw +
+                             static_cast<uint32_t>(wm * (TM * 16) + 4 * (lane >> 4));
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int v = v0 + wn * (TN * 32) + j * 32 + (lane & 31);
-        const bool v_ok = FULL || v < a.v_valid;
-        const int64_t vrow = static_cast<int64_t>(v_ok ? v : a.v_valid - 1) * a.H;
-        f32x4_t old[TM][4];
+    for (int jb = 0; jb < TN; jb += 2) {
+        f32x4_t old[2][TM];
+        bool v_ok[2];
+        int64_t vrow[2];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = jb + jj;
+            const int v = v0 + wn * (TN * 16) + AT::col(j, lane);
+            v_ok[jj] = FULL || v < a.v_valid;
+            vrow[jj] = static_cast<int64_t>(v_ok[jj] ? v : a.v_valid - 1) * a.H;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                old[i][q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < TM; ++i) {
+                old[jj][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
                 if (a.accumulate) {  // uniform
                     if (FULL) {
-                        const char* rowp = tile + (static_cast<size_t>(j * 32) * ldw + (i * 32 + 8 * q)) * 4u;
-                        old[i][q] = *reinterpret_cast<const f32x4_t*>(rowp + lane_el * 4u);
+                        const char* rowp = tile + (static_cast<size_t>(j * 16) * ldw + i * 16) * 4u;
+                        old[jj][i] = *reinterpret_cast<const f32x4_t*>(rowp + lane_el * 4u);
                     } else {
-                        const int h = hbase + i * 32 + 8 * q;
-                        old[i][q] = *reinterpret_cast<const f32x4_t*>(a.dw + vrow + (h < a.H ? h : 0));
+                        const int h = hbase + i * 16;
+                        old[jj][i] = *reinterpret_cast<const f32x4_t*>(a.dw + vrow[jj] + (h < a.H ? h : 0));
                     }
                 }
             }
+        }
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = jb + jj;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int h = hbase + i * 32 + 8 * q;
-                f32x4_t val{acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
-                            acc[i][j][q * 4 + 3]};
-                val = val * oscale + old[i][q];
+            for (int i = 0; i < TM; ++i) {
+                const int h = hbase + i * 16;
+                const f32x4_t val = acc[i][j] * oscale + old[jj][i];
                 if (FULL) {
-                    char* rowp = tile + (static_cast<size_t>(j * 32) * ldw + (i * 32 + 8 * q)) * 4u;
+                    char* rowp = tile + (static_cast<size_t>(j * 16) * ldw + i * 16) * 4u;
                     *reinterpret_cast<f32x4_t*>(rowp + lane_el * 4u) = val;
-                } else if (v_ok && h >= h_min && h < a.H) {  // H % 8 == 0: a quad is all-in or all-out
-                    *reinterpret_cast<f32x4_t*>(a.dw + vrow + h) = val;
+                } else if (v_ok[jj] && h >= h_min && h < a.H) {  // H % 8 == 0: a quad is all-in or all-out
+                    *reinterpret_cast<f32x4_t*>(a.dw + vrow[jj] + h) = val;
                 }
             }
+        }
     }
 }
 
 // Returns whether the tile was full (then every wavefront issued all its stores unconditionally).
-__device__ inline bool dw_epilogue(const f32x16_t (&acc)[kTM][kTN], const DwArgs& a, int vt, int h0,
+__device__ inline bool dw_epilogue(const f32x4_t (&acc)[Acc16::TM][Acc16::TN], const DwArgs& a, int vt, int h0,
                                    int h_min)
 {
     const bool full = vt * 256 + 256 <= a.v_valid && h0 + 256 <= a.H && h_min == h0;  // uniform
@@ -792,18 +829,18 @@ template <class T, int BK, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
 {
     using Gemm = TileGemm<T, true, true, BK>;
-    using Dtl = TileGemmDtl<T, true, true, BK, RLK_LW_DW>;
+    using Dtl = TileGemmDtl<T, true, true, BK, kWinDw>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     TileWalk walk(a.v_tiles * a.h_tiles, a.v_tiles, a.h_tiles);
     if (!walk.valid()) return;
     int vt, ht;
     walk.coords(false, vt, ht);
-    f32x16_t acc[kTM][kTN];
-    auto z_origin = [&](int v) { return a.dz + static_cast<int64_t>(v) * 256; };      // N rows
+    f32x4_t acc[Acc16::TM][Acc16::TN];
+    auto z_origin = [&](int v) { return a.dz + static_cast<int64_t>(v) * RLK_X_SAMETILE * 256; };      // N rows
     if constexpr (CHAIN) {
         // first hidden column of h tile `h`: the last tile is shifted back so that it ends at H
         auto h_col = [&](int h) { return min(h * 256, a.H - 256); };
-        auto h_origin = [&](int h) { return a.hidden + h_col(h); };  // M rows
+        auto h_origin = [&](int h) { return a.hidden + h_col(h) * RLK_X_SAMETILE; };  // M rows
         typename Dtl::Stream st;
         bool counted = false;
         Dtl::begin(st, Operand{h_origin(ht), a.H, 256}, Operand{z_origin(vt), a.ldz, 256}, a.tok_valid, smem);
@@ -812,9 +849,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
             int nvt = vt, nht = ht;
             if (more) walk.coords(true, nvt, nht);
             zero_acc(acc);
-            // a full tile's epilogue issues kTM * kTN * 4 unconditional stores per wavefront
-            Dtl::template tile<true, kTM * kTN * 2>(st, h_origin(nht), z_origin(nvt), acc, smem, counted);
-            if (more) Dtl::fetch_ahead(st, smem);
+            // a full tile's epilogue issues TM * TN unconditional stores per wavefront
+            Dtl::template tile<true, RLK_X_DW_YOUNGER>(st, h_origin(nht), z_origin(nvt), acc, smem, counted);
             counted = dw_epilogue(acc, a, vt, h_col(ht), ht * 256);
             if (!more) break;
             walk.advance();
@@ -915,24 +951,6 @@ __global__ void linear_logp_scales_kernel(const float* grad, int n, float inv_te
     }
 }
 
-// Hardware-contract self test of the transposing LDS read used for K-major operands: a 16 x 256
-// tile T[k][r] = k*256 + r is read exactly as TileIO<true,...>::frag does; out[l*8 + e] must equal
-// T[8*(l/32) + e][l % 32] (the MFMA operand layout).
-__global__ void selftest_transpose_read_kernel(int32_t* out)
-{
-    using IO = TileIO<true, 256, 16>;
-    __shared__ __attribute__((aligned(16))) char lds[IO::G::kBytes];
-    for (int i = threadIdx.x; i < 16 * 256; i += 64) {
-        const int k = i / 256, r = i % 256;
-        *reinterpret_cast<uint16_t*>(lds + k * IO::G::kPitch + r * 2) = static_cast<uint16_t>(k * 256 + r);
-    }
-    __syncthreads();
-    const u32x4_t f = IO::frag(lds, 0, 0);
-    const int l = threadIdx.x;
-    const uint32_t w[4] = {f.x, f.y, f.z, f.w};
-    for (int e = 0; e < 8; ++e) out[l * 8 + e] = (w[e >> 1] >> (16 * (e & 1))) & 0xffff;
-}
-
 }  // namespace rlk
 
 // ------------------------------------------------------------------------------------------- //
@@ -943,22 +961,6 @@ using namespace rlk;
 namespace {
 
 constexpr int kBK = RLK_BK;
-
-// 1: backward launches whose tiles are all full run one persistent workgroup per compute unit
-// that chains its tiles through one pipeline; 0: one workgroup per tile everywhere.
-#ifndef RLK_CHAIN
-#define RLK_CHAIN 1
-#endif
-#ifndef RLK_CHAIN_DH
-#define RLK_CHAIN_DH RLK_CHAIN
-#endif
-#ifndef RLK_CHAIN_DW
-#define RLK_CHAIN_DW RLK_CHAIN
-#endif
-// Extra elements between token rows of the dZ block (multiple of 8).
-#ifndef RLK_LDZ_PAD
-#define RLK_LDZ_PAD 0
-#endif
 
 // Forward launch plan: a pure function of (N, H, V, which kernels run).
 //   fast launch   : full vocab tiles [0, full_tiles) split n_fast ways
@@ -976,12 +978,9 @@ struct FwdPlan {
 // x 256 x H x 2 bytes) are re-read for every vocab tile and should stay inside the 256 MB
 // memory-side cache next to the weight tiles: 8 blocks up to H = 4096, 4 up to 8192, 2 beyond
 // (measured at H = 8192 with 16384 tokens and more: 8 blocks 1268 TFLOP/s).
-#ifndef RLK_PATCH8_MAX_H
-#define RLK_PATCH8_MAX_H 4096  // largest hidden size that keeps 8 token blocks per patch
-#endif
 int patch_rows_for(int H)
 {
-    return H <= RLK_PATCH8_MAX_H ? 8 : (H <= 2 * RLK_PATCH8_MAX_H ? 4 : 2);
+    return H <= 4096 ? 8 : (H <= 8192 ? 4 : 2);
 }
 
 int split_count(int row_blocks, int tiles, int patch_rows)
@@ -1132,7 +1131,7 @@ BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
     p.v_piece = static_cast<int>(best_pt) * 256;
     p.n_chunks = static_cast<int>((n_t + best_ct - 1) / best_ct);
     p.n_pieces = static_cast<int>((v_t + best_pt - 1) / best_pt);
-    p.ldz = p.v_piece + RLK_LDZ_PAD;
+    p.ldz = p.v_piece;
     p.dz_bytes = static_cast<size_t>(p.tok_chunk) * p.ldz * 2;
     p.acc_bytes = p.n_pieces > 1 ? static_cast<size_t>(p.tok_chunk) * H * 4 : 0;
     p.scales_off = 0;
@@ -1245,7 +1244,7 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
     using GZ = TileGemm<T, false, false, kBK>;
     using GH = TileGemm<T, true, false, kBK>;
     using GW = TileGemm<T, true, true, kBK>;
-    constexpr int kChainSmem = TileGemmDtl<T, false, false, kBK>::kSmemBytes;
+    constexpr int kChainSmem = TileGemmDtl<T, false, false, kBK, 32>::kSmemBytes;
     constexpr int kDzChainSmem = kChainSmem + kDzStageBytes * (kThreads / 64);
     const int H = c.H;
     const int64_t N = c.N, V = c.V;
@@ -1343,7 +1342,7 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
                 z.v_tiles = fast_tiles;
                 z.v_tile_lo = 0;
                 const int tiles = tok_tiles * fast_tiles;
-                if (RLK_CHAIN && k_ok && tok_valid % 256 == 0)
+                if (k_ok && tok_valid % 256 == 0)
                     hipLaunchKernelGGL((linear_logp_dz_kernel<T, kBK, false, true>),
                                        dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kDzChainSmem,
                                        stream, z);
@@ -1360,7 +1359,7 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             }
             if (dh) {
                 const int tiles = tok_tiles * h_tiles;
-                if (RLK_CHAIN_DH && p.ksplit == 1 && H >= 256 && v_valid % kBK == 0 && v_valid >= 2 * kBK) {
+                if (p.ksplit == 1 && H >= 256 && v_valid % kBK == 0 && v_valid >= 2 * kBK) {
                     hipLaunchKernelGGL((linear_logp_dh_kernel<T, kBK, true>),
                                        dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kChainSmem,
                                        stream, h);
@@ -1378,7 +1377,7 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             }
             if (c.d_weight) {
                 const int tiles = v_tiles * h_tiles;
-                if (RLK_CHAIN_DW && H >= 256 && tok_valid % kBK == 0 && tok_valid >= 2 * kBK)
+                if (H >= 256 && tok_valid % kBK == 0 && tok_valid >= 2 * kBK)
                     hipLaunchKernelGGL((linear_logp_dw_kernel<T, kBK, true>),
                                        dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kChainSmem,
                                        stream, d);
@@ -1717,13 +1716,6 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
 }  // namespace
 
 extern "C" {
-
-int rlk_selftest_transpose_read(int32_t* out, hipStream_t stream)
-{
-    if (!out) return rlk_fail(RLK_ERR_ARG, "null pointer");
-    hipLaunchKernelGGL(selftest_transpose_read_kernel, dim3(1), dim3(64), 0, stream, out);
-    return check_launch("selftest launch failed");
-}
 
 int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                         size_t dz_budget_bytes, size_t* bytes)

@@ -366,7 +366,7 @@ __global__ __launch_bounds__(kThreads) void wide_fwd_kernel(WideFwdArgs a)
         f32x16_t acc[kTM][kTN];
         zero_acc(acc);
         Gemm::run(A, B, a.H, acc, smem);
-        fwd_epilogue<true>(acc, a, a.bias, v0 + wm * (kTM * 32), lane, tgt, m, s, zt);
+        fwd_epilogue<true, Acc32>(acc, a, a.bias, v0 + wm * (kTM * 32), lane, tgt, m, s, zt);
     }
 
     // merge: the two half-wave row groups of a token, then the wavefronts along M (fixed order)
