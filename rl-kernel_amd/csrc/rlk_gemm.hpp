@@ -471,15 +471,10 @@ struct DtlIO {
         const char* src = (over ? next : base) + static_cast<size_t>(rel) * step;
         const uint32_t dst = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
                                  (RLK_LDS char*)(lds))) + static_cast<uint32_t>((wave + kWaves * p) * 1024);
-#ifndef RLK_X_NOLOAD
         asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                      :
                      : "v"(off[p]), "s"(src), "s"(dst)
                      : "memory", "m0");
-#else
-        (void)src;
-        (void)dst;
-#endif
     }
 
     // MFMA 16x16x32 operand fragment: lane l holds row (row0 + l%16), k = kk*32 + 8*(l/16) + 0..7

@@ -15,42 +15,13 @@
 #include "rlk_tile_epilogue.hpp"
 
 // Load windows (MFMA slots of a K step's second slice over which its 8 loads are spread, see
-// TileGemmDtl), measured one kernel at a time at the Llama head: the persistent dZ and dH kernels
-// are faster with all loads out early, the forward and dW with the loads spread over the slice.
-#ifndef RLK_X_WIN_FWD
-#define RLK_X_WIN_FWD 32
-#endif
-#ifndef RLK_X_WIN_DZ
-#define RLK_X_WIN_DZ 16
-#endif
-#ifndef RLK_X_WIN_DH
-#define RLK_X_WIN_DH 16
-#endif
-#ifndef RLK_X_WIN_DW
-#define RLK_X_WIN_DW 32
-#endif
-#ifndef RLK_X_FWD_REFETCH
-#define RLK_X_FWD_REFETCH false
-#endif
-#ifndef RLK_X_DZ_YOUNGER
-#define RLK_X_DZ_YOUNGER 0
-#endif
-#ifndef RLK_X_SAMETILE
-#define RLK_X_SAMETILE 1  // experiment: 0 = every workgroup fetches tile 0 (all loads hit L2)
-#endif
-#ifndef RLK_X_DH_YOUNGER
-#define RLK_X_DH_YOUNGER (Acc16::TM * Acc16::TN / 2)
-#endif
-#ifndef RLK_X_DW_YOUNGER
-#define RLK_X_DW_YOUNGER (Acc16::TM * Acc16::TN / 2)
-#endif
-constexpr int kWinFwd = RLK_X_WIN_FWD;
-constexpr int kWinDz = RLK_X_WIN_DZ;
-constexpr int kWinDh = RLK_X_WIN_DH;
-constexpr int kWinDw = RLK_X_WIN_DW;
-// The forward carries the first fragments of the next tile through the softmax update (false) or
-// reads them again from LDS afterwards (true).
-constexpr bool kFwdRefetch = RLK_X_FWD_REFETCH;
+// TileGemmDtl), measured one kernel at a time at the Llama head (launch time with 16 / 24 / 32
+// slots: dZ 791 / 801 / 819 us, dH 822 / 813 / 799 us, dW 866 / 852 / 846 us; forward 23.71 / 23.64 /
+// 23.63 ms).
+constexpr int kWinFwd = 32;
+constexpr int kWinDz = 16;
+constexpr int kWinDh = 32;
+constexpr int kWinDw = 32;
 
 namespace rlk {
 
@@ -204,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_fwd_kernel(FwdArgs a)
                 const void* next = vt + 1 < t1 ? tile_origin(head, vt + 1)
                                                : (head + 1 < n_heads ? tile_origin(head + 1, t0)
                                                                      : tile_origin(head, vt));
-                Dtl::template tile<kFwdRefetch>(st, next, B.base, acc, smem);
+                Dtl::template tile<true>(st, next, B.base, acc, smem);
                 const float* bias = head == 0 ? a.bias : a.bias2;
                 if (bias != nullptr) add_bias<AT>(acc, bias, vt * 256 + wm * (TM * 16), lane);  // uniform
                 fwd_epilogue<GENERAL, AT>(acc, a, nullptr, vt * 256 + wm * (TM * 16), lane, tgt, m, s, zt);
@@ -360,8 +331,6 @@ struct DzArgs {
 // LDS each wavefront needs to turn its part of a dZ tile into full rows: 64 tokens x 32 vocab
 // columns of 16-bit values, 64 bytes per token row, no padding.
 constexpr int kDzStageBytes = 64 * 64;
-// Global stores one wavefront issues per dZ tile (four 32-row groups x 8 row batches), all unconditional.
-constexpr int kDzStores = (Acc16::TM / 2) * 8;
 
 // dZ epilogue of one 256 x 256 tile.  A wavefront owns 128 vocab rows x 64 tokens of the tile; for
 // each of its four 32-row groups (two 16-row MFMA tiles) it writes the rounded values into its
@@ -478,8 +447,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
     if (!walk.valid()) return;
     int vt, tt;
     walk.coords(false, vt, tt);
-    auto w_origin = [&](int v) { return a.weight + static_cast<int64_t>(v + a.v_tile_lo) * RLK_X_SAMETILE * 256 * a.H; };
-    auto h_origin = [&](int t) { return a.hidden + static_cast<int64_t>(t) * RLK_X_SAMETILE * 256 * a.H; };
+    auto w_origin = [&](int v) { return a.weight + static_cast<int64_t>(v + a.v_tile_lo) * 256 * a.H; };
+    auto h_origin = [&](int t) { return a.hidden + static_cast<int64_t>(t) * 256 * a.H; };
     f32x4_t acc[AT::TM][AT::TN];
     if constexpr (CHAIN) {
         char* stage = smem + Dtl::kSmemBytes + wave * kDzStageBytes;
@@ -490,7 +459,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dz_kernel(DzArgs a)
             int nvt = vt, ntt = tt;
             if (more) walk.coords(true, nvt, ntt);
             zero_acc(acc);
-            Dtl::template tile<true, RLK_X_DZ_YOUNGER>(st, w_origin(nvt), h_origin(ntt), acc, smem, true);
+            Dtl::template tile<true>(st, w_origin(nvt), h_origin(ntt), acc, smem);
             if (a.bias != nullptr)  // uniform
                 add_bias<AT>(acc, a.bias, (vt + a.v_tile_lo) * 256 + (wave / kWN) * (AT::TM * 16), threadIdx.x & 63);
             dz_epilogue<T, GENERAL>(acc, a, vt + a.v_tile_lo, tt, stage);
@@ -649,8 +618,8 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
         walk.coords(false, tt, ht);
         // first hidden column of h tile `h`: the last tile is shifted back so that it ends at H
         auto h_col = [&](int h) { return min(h * 256, a.H - 256); };
-        auto w_origin = [&](int h) { return a.weight + h_col(h) * RLK_X_SAMETILE; };
-        auto z_origin = [&](int t) { return a.dz + static_cast<int64_t>(t) * RLK_X_SAMETILE * 256 * a.ldz; };
+        auto w_origin = [&](int h) { return a.weight + h_col(h); };
+        auto z_origin = [&](int t) { return a.dz + static_cast<int64_t>(t) * 256 * a.ldz; };
         typename Dtl::Stream st;
         bool counted = false;
         Dtl::begin(st, Operand{w_origin(ht), a.H, 256}, Operand{z_origin(tt), a.ldz, 256}, a.v_valid, smem);
@@ -660,7 +629,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dh_kernel(DhArgs a)
             if (more) walk.coords(true, ntt, nht);
             zero_acc(acc);
             // a full tile's epilogue issues TM * TN unconditional stores per wavefront
-            Dtl::template tile<true, RLK_X_DH_YOUNGER>(st, w_origin(nht), z_origin(ntt), acc, smem, counted);
+            Dtl::template tile<true, Acc16::TM * Acc16::TN / 2>(st, w_origin(nht), z_origin(ntt), acc, smem, counted);
             counted = dh_epilogue<T>(acc, a, tt, h_col(ht), ht * 256, a.acc, a.first != 0, a.last != 0);
             if (!more) break;
             walk.advance();
@@ -836,11 +805,11 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
     int vt, ht;
     walk.coords(false, vt, ht);
     f32x4_t acc[Acc16::TM][Acc16::TN];
-    auto z_origin = [&](int v) { return a.dz + static_cast<int64_t>(v) * RLK_X_SAMETILE * 256; };      // N rows
+    auto z_origin = [&](int v) { return a.dz + static_cast<int64_t>(v) * 256; };      // N rows
     if constexpr (CHAIN) {
         // first hidden column of h tile `h`: the last tile is shifted back so that it ends at H
         auto h_col = [&](int h) { return min(h * 256, a.H - 256); };
-        auto h_origin = [&](int h) { return a.hidden + h_col(h) * RLK_X_SAMETILE; };  // M rows
+        auto h_origin = [&](int h) { return a.hidden + h_col(h); };  // M rows
         typename Dtl::Stream st;
         bool counted = false;
         Dtl::begin(st, Operand{h_origin(ht), a.H, 256}, Operand{z_origin(vt), a.ldz, 256}, a.tok_valid, smem);
@@ -850,7 +819,7 @@ __global__ __launch_bounds__(kThreads) void linear_logp_dw_kernel(DwArgs a)
             if (more) walk.coords(true, nvt, nht);
             zero_acc(acc);
             // a full tile's epilogue issues TM * TN unconditional stores per wavefront
-            Dtl::template tile<true, RLK_X_DW_YOUNGER>(st, h_origin(nht), z_origin(nvt), acc, smem, counted);
+            Dtl::template tile<true, Acc16::TM * Acc16::TN / 2>(st, h_origin(nht), z_origin(nvt), acc, smem, counted);
             counted = dw_epilogue(acc, a, vt, h_col(ht), ht * 256);
             if (!more) break;
             walk.advance();
