@@ -160,6 +160,23 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                         int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
                         int64_t ignore_index, int32_t use_ignore, rlk_stream_t stream);
 
+/* rlk_linear_logp_bwd into a running fp32 gradient: with accumulate != 0, d_weight and d_bias are
+ * ADDED to what the buffers hold (d_weight += dZ^T H, d_bias += sum_n dZ) instead of overwritten;
+ * accumulate == 0 is rlk_linear_logp_bwd.  d_hidden is always overwritten.  This is the reference's
+ * own accumulation pattern moved to the caller's buffer: chunked_linear_logp_backward keeps one
+ * fp32 grad_w over all token chunks and casts once at the end
+ * (rl_engine/kernels/ops/pytorch/loss/linear_logp.py:404,423-437).  A trainer that keeps fp32 main
+ * gradients hands that buffer in and runs micro-batch after micro-batch into it: no [V, H]
+ * temporary and no cast per call.  The sum over micro-batches is taken in call order (stream
+ * order), so it is as repeatable as the calls. */
+int rlk_linear_logp_bwd_accum(const float* grad_logp, const void* hidden, const void* weight,
+                              const float* bias, const int64_t* targets, const float* lse,
+                              void* d_hidden, float* d_weight, float* d_bias, void* workspace,
+                              size_t workspace_bytes, size_t dz_budget_bytes, int64_t N, int32_t H,
+                              int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                              int64_t ignore_index, int32_t use_ignore, int32_t accumulate,
+                              rlk_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------ *
  * Final RMSNorm in front of the head (the step before the path).
  *

@@ -1119,12 +1119,30 @@ BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
     return p;
 }
 
+// Raises the dynamic-LDS limit of `kernel` to `bytes` on the current device.  The attribute is
+// per device and sticks, so each (kernel instance, device) pair pays the runtime call once.
 template <class K>
 int set_smem(K kernel, int bytes)
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    return e == hipSuccess ? 0 : rlk_fail(RLK_ERR_LAUNCH, hipGetErrorString(e));
+    constexpr int kMaxDev = 64;
+    static std::mutex mu;
+    static int done[kMaxDev] = {};  // one table per template instance = per kernel
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, hipGetErrorString(e));
+    const bool tracked = dev >= 0 && dev < kMaxDev;
+    if (tracked) {
+        std::lock_guard<std::mutex> lock(mu);
+        if (done[dev] >= bytes) return 0;
+    }
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return rlk_fail(RLK_ERR_LAUNCH, hipGetErrorString(e));
+    if (tracked) {
+        std::lock_guard<std::mutex> lock(mu);
+        if (done[dev] < bytes) done[dev] = bytes;
+    }
+    return 0;
 }
 
 int check_launch(const char* what)
@@ -1724,6 +1742,20 @@ int rlk_linear_logp_bwd(const float* grad_logp, const void* hidden, const void* 
                                              d_weight, d_bias, workspace, workspace_bytes,
                                              dz_budget_bytes, N, H, V, vocab_start, dtype, temperature,
                                              ignore_index, use_ignore, 0, stream);
+}
+
+int rlk_linear_logp_bwd_accum(const float* grad_logp, const void* hidden, const void* weight,
+                              const float* bias, const int64_t* targets, const float* lse,
+                              void* d_hidden, float* d_weight, float* d_bias, void* workspace,
+                              size_t workspace_bytes, size_t dz_budget_bytes, int64_t N, int32_t H,
+                              int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
+                              int64_t ignore_index, int32_t use_ignore, int32_t accumulate,
+                              hipStream_t stream)
+{
+    return rlk::linear_logp_bwd_accumulating(grad_logp, hidden, weight, bias, targets, lse, d_hidden,
+                                             d_weight, d_bias, workspace, workspace_bytes,
+                                             dz_budget_bytes, N, H, V, vocab_start, dtype, temperature,
+                                             ignore_index, use_ignore, accumulate != 0 ? 1 : 0, stream);
 }
 
 }  // extern "C"

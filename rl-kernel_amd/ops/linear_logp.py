@@ -45,6 +45,15 @@ def _out_of_range_error(target_1d: torch.Tensor, vocab: int, ignore_index: Optio
     )
 
 
+def _check_grad_buffer(name: str, buf: torch.Tensor, shape, device) -> None:
+    if buf.dtype != torch.float32 or tuple(buf.shape) != tuple(shape) or not buf.is_contiguous() \
+            or buf.device != device:
+        raise ValueError(f"{name} must be a contiguous float32 tensor of shape {tuple(shape)} on "
+                         f"{device}, got {buf.dtype} {tuple(buf.shape)} on {buf.device}")
+    if buf.requires_grad:
+        raise ValueError(f"{name} must not require grad (it is a gradient buffer)")
+
+
 def hip_path_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     """bf16 / f16 / f32 tensors of one dtype on one GPU.  bf16/f16 with a hidden size that is a
     multiple of 8 run on the 16-bit MFMA tiles, the rest on the fp32 matrix-core kernels."""
@@ -279,12 +288,20 @@ def fused_linear_logp_backward(
     need_weight: bool = True,
     need_bias: bool = True,
     dz_budget_bytes: int = 0,
+    weight_grad_out: Optional[torch.Tensor] = None,
+    bias_grad_out: Optional[torch.Tensor] = None,
+    accumulate: bool = False,
 ):
     """Raw backward: ``(d_hidden [N,H] input dtype, d_weight [V,H] fp32, d_bias [V] fp32)``.
 
     Stand-in for ``chunked_linear_logp_backward``
     (rl_engine/kernels/ops/pytorch/loss/linear_logp.py:383-439 of the reference); unlike it, the
     saved ``lse`` is used (as the vocab-parallel backward does, :313).
+
+    ``weight_grad_out`` / ``bias_grad_out``: caller-owned fp32 ``[V,H]`` / ``[V]`` buffers that
+    receive the gradients instead of fresh tensors (they are what the call returns);
+    ``accumulate`` adds to what they hold instead of overwriting it, as the reference keeps one
+    fp32 ``grad_w`` over its token chunks (same file :404,423-437).
     """
     lib = _native.load()
     n, h = hidden_2d.shape
@@ -293,32 +310,46 @@ def fused_linear_logp_backward(
     dt = _DTYPES[hidden_2d.dtype]
     g = grad_logp.reshape(-1).to(torch.float32).contiguous()
     d_hidden = torch.empty_like(hidden_2d) if need_hidden else None
-    d_weight = torch.empty(v, h, device=dev, dtype=torch.float32) if need_weight else None
     want_bias = bias is not None and need_bias
-    d_bias = torch.empty(v, device=dev, dtype=torch.float32) if want_bias else None
+    if weight_grad_out is not None:
+        _check_grad_buffer("weight_grad_out", weight_grad_out, (v, h), dev)
+    if bias_grad_out is not None:
+        _check_grad_buffer("bias_grad_out", bias_grad_out, (v,), dev)
+    if accumulate and ((need_weight and weight_grad_out is None) or (want_bias and bias_grad_out is None)):
+        raise ValueError("accumulate=True needs the buffers to add to (weight_grad_out / bias_grad_out)")
+    d_weight = None
+    if need_weight:
+        d_weight = weight_grad_out if weight_grad_out is not None else \
+            torch.empty(v, h, device=dev, dtype=torch.float32)
+    d_bias = None
+    if want_bias:
+        d_bias = bias_grad_out if bias_grad_out is not None else \
+            torch.empty(v, device=dev, dtype=torch.float32)
     bias_f = None if bias is None else bias.detach().to(torch.float32).contiguous()
     need = _native.ctypes.c_size_t(0)
     _native.check(lib.rlk_linear_logp_bwd_workspace_bytes(n, h, v, dt, int(dz_budget_bytes),
                                                           _native.ctypes.byref(need)),
                   "linear_logp backward workspace query")
     ws = torch.empty(need.value, device=dev, dtype=torch.uint8)
-    rc = lib.rlk_linear_logp_bwd(
+    rc = lib.rlk_linear_logp_bwd_accum(
         _ptr(g), _ptr(hidden_2d), _ptr(weight), _ptr(bias_f), _ptr(target_1d), _ptr(lse),
         _ptr(d_hidden), _ptr(d_weight), _ptr(d_bias), _ptr(ws), ws.numel(), int(dz_budget_bytes),
         n, h, v, int(vocab_start), dt, float(temperature),
         0 if ignore_index is None else int(ignore_index), int(ignore_index is not None),
-        _stream(dev))
-    _native.check(rc, "rlk_linear_logp_bwd")
+        int(bool(accumulate)), _stream(dev))
+    _native.check(rc, "rlk_linear_logp_bwd_accum")
     return d_hidden, d_weight, d_bias
 
 
 class _FusedLinearLogpFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, bias, target_ids, temperature, ignore_index, check_targets):
+    def forward(ctx, hidden, weight, bias, target_ids, temperature, ignore_index, check_targets,
+                weight_grad_out=None, bias_grad_out=None, accumulate=True):
         hidden_2d = _aligned_contiguous(hidden.reshape(-1, hidden.size(-1)))
         w = _aligned_contiguous(weight)
         target_1d = target_ids.reshape(-1).to(device=hidden_2d.device, dtype=torch.long).contiguous()
         ctx.empty = hidden_2d.size(0) == 0
+        ctx.weight_grad_out, ctx.bias_grad_out, ctx.accumulate = weight_grad_out, bias_grad_out, accumulate
         if ctx.empty:  # no tokens: nothing to launch, gradients are zeros
             ctx.save_for_backward(hidden_2d, w, bias if bias is not None else hidden_2d, target_1d,
                                   hidden_2d.new_zeros(0, dtype=torch.float32))
@@ -345,19 +376,42 @@ class _FusedLinearLogpFunction(torch.autograd.Function):
         hidden_2d, w, bias_t, target_1d, lse = ctx.saved_tensors
         need_h, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[1], \
             ctx.has_bias and ctx.needs_input_grad[2]
+        w_out = getattr(ctx, "weight_grad_out", None)
+        b_out = getattr(ctx, "bias_grad_out", None)
+        accumulate = getattr(ctx, "accumulate", True)
+        nones = (None,) * 7
         if ctx.empty:
+            # no tokens: the gradients are zeros; buffers that accumulate stay as they are
+            if w_out is not None and not accumulate:
+                w_out.zero_()
+            if b_out is not None and not accumulate:
+                b_out.zero_()
             return (hidden_2d.new_zeros(tuple(ctx.lead_shape) + (hidden_2d.size(1),)) if need_h else None,
-                    torch.zeros_like(w, dtype=ctx.weight_dtype) if need_w else None,
-                    torch.zeros_like(bias_t, dtype=ctx.bias_dtype) if need_b else None,
-                    None, None, None, None)
+                    torch.zeros_like(w, dtype=ctx.weight_dtype) if need_w and w_out is None else None,
+                    torch.zeros_like(bias_t, dtype=ctx.bias_dtype) if need_b and b_out is None else None,
+                    *nones)
+        # a caller-owned buffer receives its gradient even when the parameter itself is frozen for
+        # autograd (main-grad trainers detach their parameters' .grad handling)
+        want_w = need_w or w_out is not None
+        want_b = ctx.has_bias and (need_b or b_out is not None)
+        adding = accumulate and (w_out is not None or b_out is not None)
+        w_buf, b_buf = w_out, b_out
+        if adding:
+            # one switch covers both buffers in the library: a gradient without a caller buffer
+            # gets a zeroed one here, so that adding to it is the same as writing it
+            if want_w and w_buf is None:
+                w_buf = torch.zeros(w.shape, device=w.device, dtype=torch.float32)
+            if want_b and b_buf is None:
+                b_buf = torch.zeros(w.size(0), device=w.device, dtype=torch.float32)
         d_h, d_w, d_b = fused_linear_logp_backward(
             grad_logp, hidden_2d, w, target_1d, lse, bias_t if ctx.has_bias else None,
             temperature=ctx.temperature, ignore_index=ctx.ignore_index,
-            need_hidden=need_h, need_weight=need_w, need_bias=need_b)
+            need_hidden=need_h, need_weight=want_w, need_bias=want_b,
+            weight_grad_out=w_buf, bias_grad_out=b_buf, accumulate=adding)
         grad_hidden = d_h.reshape(tuple(ctx.lead_shape) + (hidden_2d.size(1),)) if need_h else None
-        grad_weight = d_w.to(ctx.weight_dtype) if need_w else None
-        grad_bias = d_b.to(ctx.bias_dtype) if need_b else None
-        return grad_hidden, grad_weight, grad_bias, None, None, None, None
+        grad_weight = d_w.to(ctx.weight_dtype) if need_w and w_out is None else None
+        grad_bias = d_b.to(ctx.bias_dtype) if need_b and b_out is None else None
+        return (grad_hidden, grad_weight, grad_bias, *nones)
 
 
 class _FusedNormLinearLogpFunction(torch.autograd.Function):
@@ -454,18 +508,31 @@ class RocmFusedLinearLogpOp:
                  vocab_start_index: int = 0, global_vocab_size: Optional[int] = None,
                  temperature: float = 1.0, ignore_index: Optional[int] = None,
                  check_targets: bool = True, norm_weight: Optional[torch.Tensor] = None,
-                 norm_eps: float = 1e-6) -> torch.Tensor:
+                 norm_eps: float = 1e-6, weight_grad_out: Optional[torch.Tensor] = None,
+                 bias_grad_out: Optional[torch.Tensor] = None,
+                 accumulate: bool = True) -> torch.Tensor:
         return self.apply(hidden, lm_head_weight, target_ids, bias, tp_group=tp_group,
                           vocab_start_index=vocab_start_index, global_vocab_size=global_vocab_size,
                           temperature=temperature, ignore_index=ignore_index,
-                          check_targets=check_targets, norm_weight=norm_weight, norm_eps=norm_eps)
+                          check_targets=check_targets, norm_weight=norm_weight, norm_eps=norm_eps,
+                          weight_grad_out=weight_grad_out, bias_grad_out=bias_grad_out,
+                          accumulate=accumulate)
 
     def apply(self, hidden, lm_head_weight, target_ids, bias=None, *, tp_group: Any = None,
               vocab_start_index: int = 0, global_vocab_size: Optional[int] = None,
               temperature: float = 1.0, ignore_index: Optional[int] = None,
               check_targets: bool = True, norm_weight: Optional[torch.Tensor] = None,
-              norm_eps: float = 1e-6) -> torch.Tensor:
+              norm_eps: float = 1e-6, weight_grad_out: Optional[torch.Tensor] = None,
+              bias_grad_out: Optional[torch.Tensor] = None, accumulate: bool = True) -> torch.Tensor:
         """Selected-token log-prob in float32 with the leading shape of ``hidden``.
+
+        ``weight_grad_out`` / ``bias_grad_out`` (keyword-only, default off): contiguous float32
+        ``[V, H]`` / ``[V]`` buffers of the caller (fp32 main gradients).  The backward then adds
+        the head's weight / bias gradient to them in place (``accumulate=False``: overwrites them)
+        and autograd returns ``None`` for that parameter: no ``[V, H]`` temporary and no cast per
+        call, and micro-batches accumulate as the reference's backward accumulates its token
+        chunks into one fp32 ``grad_w``
+        (rl_engine/kernels/ops/pytorch/loss/linear_logp.py:404,423-437 of the reference).
 
         ``norm_weight`` (keyword-only, default off): ``hidden`` is then the UN-normalised output
         of the last layer and the model's final RMSNorm
@@ -513,7 +580,16 @@ class RocmFusedLinearLogpOp:
             raise NotImplementedError(
                 "RocmFusedLinearLogpOp needs hidden and lm_head_weight in bf16, f16 or f32 on the "
                 "same GPU (and of one dtype when norm_weight is given)")
+        for name, buf, shape in (("weight_grad_out", weight_grad_out, tuple(lm_head_weight.shape)),
+                                 ("bias_grad_out", bias_grad_out, (vocab,))):
+            if buf is not None:
+                _check_grad_buffer(name, buf, shape, hidden.device)
+        if bias_grad_out is not None and bias is None:
+            raise ValueError("bias_grad_out given without a bias")
         if norm_weight is not None:
+            if weight_grad_out is not None or bias_grad_out is not None:
+                raise NotImplementedError("weight_grad_out / bias_grad_out are not wired into the "
+                                          "norm_weight form of the op")
             if norm_weight.dim() != 1 or norm_weight.shape[0] != hidden.size(-1):
                 raise ValueError(f"norm_weight must be 1-D of size hidden.shape[-1]={hidden.size(-1)}, "
                                  f"got tuple(norm_weight.shape)={tuple(norm_weight.shape)}")
@@ -524,7 +600,8 @@ class RocmFusedLinearLogpOp:
                                                       target_ids, float(norm_eps), float(temperature),
                                                       ignore_index, check_targets)
         return _FusedLinearLogpFunction.apply(hidden, lm_head_weight, bias, target_ids,
-                                              float(temperature), ignore_index, check_targets)
+                                              float(temperature), ignore_index, check_targets,
+                                              weight_grad_out, bias_grad_out, bool(accumulate))
 
     def with_reference(self, hidden, lm_head_weight, ref_lm_head_weight, target_ids, bias=None,
                        ref_bias=None, *, temperature: float = 1.0,
