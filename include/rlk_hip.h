@@ -183,17 +183,19 @@ int rlk_linear_logp_bwd_accum(const float* grad_logp, const void* hidden, const 
  * rlk_rmsnorm_fwd stands in for NativeRMSNormOp.forward
  * (rl_engine/kernels/ops/pytorch/norm/rms_norm.py:28-70):
  *   out = cast_to_dtype( (x * rsqrt(mean(x^2, -1) + eps)) * gain ),  fp32 arithmetic,
- * x / out [N, H] and gain [H] of `dtype` (bf16 / f16 / f32), rstd [N] f32 optional.  A row's
+ * x / out [N, H] of `dtype` (bf16 / f16 / f32), gain [H] ALWAYS f32 (the reference multiplies by
+ * weight.float(), :66-70, so a gain kept in fp32 over 16-bit activations loses nothing), rstd [N]
+ * f32 optional.  A row's
  * result does not depend on the other rows of the batch.  rlk_rmsnorm_bwd is its backward
  * (what autograd derives for that expression): d_x [N, H] of `dtype`, d_gain [H] f32
  * (overwritten; NULL to skip) from d_out [N, H] of `dtype`; the row statistics are recomputed.
  * ------------------------------------------------------------------------------------------ */
-int rlk_rmsnorm_fwd(const void* x, const void* gain, float eps, void* out, float* rstd, int64_t N,
+int rlk_rmsnorm_fwd(const void* x, const float* gain, float eps, void* out, float* rstd, int64_t N,
                     int32_t H, int32_t dtype, rlk_stream_t stream);
 
 int rlk_rmsnorm_bwd_workspace_bytes(int64_t N, int32_t H, size_t* bytes);
 
-int rlk_rmsnorm_bwd(const void* x, const void* gain, float eps, const void* d_out, void* d_x,
+int rlk_rmsnorm_bwd(const void* x, const float* gain, float eps, const void* d_out, void* d_x,
                     float* d_gain, void* workspace, size_t workspace_bytes, int64_t N, int32_t H,
                     int32_t dtype, rlk_stream_t stream);
 
@@ -202,16 +204,19 @@ int rlk_rmsnorm_bwd(const void* x, const void* gain, float eps, const void* d_ou
  * UN-normalised hidden states x and the norm gain.
  *   forward : logp / lse of  linear_logp( rmsnorm(x, gain, eps), weight, bias, ... ),
  *             bit for bit what rlk_rmsnorm_fwd followed by rlk_linear_logp_fwd return on the same
- *             blocks of 32768 tokens (the whole input when N <= 32768);
+ *             blocks of 8192 tokens (the whole input when N <= 8192);
  *   backward: d_x (gradient w.r.t. the un-normalised hidden states, `dtype`), d_gain [H] f32,
  *             d_weight [V, H] f32, d_bias [V] f32 -- rlk_linear_logp_bwd followed by rlk_rmsnorm_bwd.
- * The normalised rows are never saved: they exist as one block of at most 32768 tokens inside the
- * workspace in either direction (the backward recomputes them), so the caller keeps only x, and the
- * extra memory stays independent of N.  Any gradient pointer may be NULL. */
+ * The normalised rows are never saved: they exist as one block of at most 8192 tokens (64 MiB of
+ * 16-bit rows at H = 4096) inside the workspace in either direction (the backward recomputes them),
+ * so the caller keeps only x, and the extra memory stays independent of N.  In the backward the
+ * head's gradient w.r.t. the normalised rows is written into the caller's d_x and the norm backward
+ * runs on it in place.  Any gradient pointer may be NULL (without d_x the blocks are half as long
+ * and the second half of the row region holds that gradient). */
 int rlk_linear_logp_rmsnorm_fwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                                 size_t* bytes);
 
-int rlk_linear_logp_rmsnorm_fwd(const void* x, const void* gain, float eps, const void* weight,
+int rlk_linear_logp_rmsnorm_fwd(const void* x, const float* gain, float eps, const void* weight,
                                 const float* bias, const int64_t* targets, float* logp, float* lse,
                                 void* workspace, size_t workspace_bytes, int64_t N, int32_t H,
                                 int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
@@ -221,7 +226,7 @@ int rlk_linear_logp_rmsnorm_fwd(const void* x, const void* gain, float eps, cons
 int rlk_linear_logp_rmsnorm_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                                 size_t dz_budget_bytes, size_t* bytes);
 
-int rlk_linear_logp_rmsnorm_bwd(const float* grad_logp, const void* x, const void* gain, float eps,
+int rlk_linear_logp_rmsnorm_bwd(const float* grad_logp, const void* x, const float* gain, float eps,
                                 const void* weight, const float* bias, const int64_t* targets,
                                 const float* lse, void* d_x, float* d_gain, float* d_weight,
                                 float* d_bias, void* workspace, size_t workspace_bytes,

@@ -11,6 +11,7 @@ constexpr int kNormThreads = 256;
 constexpr int kNormRowsPerGroup = 64;  // rows one workgroup of the backward walks (d_gain partial)
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4n;
+typedef __attribute__((ext_vector_type(4))) float f32x4n;
 
 template <int DT>
 struct NormElem;
@@ -78,33 +79,32 @@ __device__ inline float row_sum_squares(const typename NormElem<DT>::type* x, in
     return norm_block_sum(ss);
 }
 
-// One workgroup per row: rstd = rsqrt(mean(x^2) + eps); out = cast((x * rstd) * gain).
+// One workgroup per row: rstd = rsqrt(mean(x^2) + eps); out = cast((x * rstd) * gain), gain in fp32.
 template <int DT, int VEC>
-__global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_kernel(const void* x_v, const void* gain_v,
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_kernel(const void* x_v, const float* gain,
                                                                    float eps, void* out_v, float* rstd,
                                                                    int H)
 {
     using E = typename NormElem<DT>::type;
     const int64_t row = blockIdx.x;
     const E* x = static_cast<const E*>(x_v) + row * H;
-    const E* gain = static_cast<const E*>(gain_v);
     E* out = static_cast<E*>(out_v) + row * H;
     const float r = rsqrtf(row_sum_squares<DT, VEC>(x, H) / static_cast<float>(H) + eps);
     if (rstd != nullptr && threadIdx.x == 0) rstd[row] = r;
     for (int h = threadIdx.x * VEC; h < H; h += kNormThreads * VEC) {
         if constexpr (VEC == 8) {
             const u32x4n xv = *reinterpret_cast<const u32x4n*>(x + h);
-            const u32x4n gv = *reinterpret_cast<const u32x4n*>(gain + h);
+            const f32x4n g0 = *reinterpret_cast<const f32x4n*>(gain + h);
+            const f32x4n g1 = *reinterpret_cast<const f32x4n*>(gain + h + 4);
+            const float ge[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
             const E* xe = reinterpret_cast<const E*>(&xv);
-            const E* ge = reinterpret_cast<const E*>(&gv);
             u32x4n ov;
             E* oe = reinterpret_cast<E*>(&ov);
 #pragma unroll
-            for (int k = 0; k < 8; ++k)
-                oe[k] = NormElem<DT>::put((NormElem<DT>::get(xe[k]) * r) * NormElem<DT>::get(ge[k]));
+            for (int k = 0; k < 8; ++k) oe[k] = NormElem<DT>::put((NormElem<DT>::get(xe[k]) * r) * ge[k]);
             *reinterpret_cast<u32x4n*>(out + h) = ov;
         } else {
-            out[h] = NormElem<DT>::put((NormElem<DT>::get(x[h]) * r) * NormElem<DT>::get(gain[h]));
+            out[h] = NormElem<DT>::put((NormElem<DT>::get(x[h]) * r) * gain[h]);
         }
     }
 }
@@ -115,14 +115,13 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_kernel(const void* x
 // ascending order) and written as one partial row; rmsnorm_gain_finish_kernel adds the partials
 // in group order.
 template <int DT, int VEC>
-__global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const void* x_v, const void* gain_v,
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const void* x_v, const float* gain,
                                                                    float eps, const void* dout_v,
                                                                    void* dx_v, float* gain_part,
                                                                    int64_t n_rows, int H)
 {
     using E = typename NormElem<DT>::type;
     extern __shared__ float dg[];  // [H]
-    const E* gain = static_cast<const E*>(gain_v);
     for (int h = threadIdx.x; h < H; h += kNormThreads) dg[h] = 0.f;  // (own columns only below)
     __syncthreads();
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kNormRowsPerGroup;
@@ -136,8 +135,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const void* x
         for (int h = threadIdx.x * VEC; h < H; h += kNormThreads * VEC) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k)
-                dot += (NormElem<DT>::get(dy[h + k]) * NormElem<DT>::get(gain[h + k])) *
-                       NormElem<DT>::get(x[h + k]);
+                dot += (NormElem<DT>::get(dy[h + k]) * gain[h + k]) * NormElem<DT>::get(x[h + k]);
         }
         dot = norm_block_sum(dot);
         const float c = r * r * r * dot / static_cast<float>(H);
@@ -146,7 +144,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const void* x
             for (int k = 0; k < VEC; ++k) {
                 const float xf = NormElem<DT>::get(x[h + k]);
                 const float dyf = NormElem<DT>::get(dy[h + k]);
-                const float g = dyf * NormElem<DT>::get(gain[h + k]);
+                const float g = dyf * gain[h + k];
                 dx[h + k] = NormElem<DT>::put(r * g - xf * c);
                 dg[h + k] += dyf * xf * r;
             }
@@ -178,7 +176,7 @@ bool vec_ok(const void* a, const void* b, const void* c, int H, int dtype)
     return dtype != RLK_DTYPE_F32 && H % 8 == 0 && (bits & 15) == 0;
 }
 
-int check_norm(const void* x, const void* gain, int64_t N, int32_t H, int dtype)
+int check_norm(const void* x, const float* gain, int64_t N, int32_t H, int dtype)
 {
     if (!x || !gain) return rlk_fail(RLK_ERR_ARG, "null pointer");
     if (N <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "N and H must be positive");
@@ -190,7 +188,7 @@ int check_norm(const void* x, const void* gain, int64_t N, int32_t H, int dtype)
 }
 
 template <int DT>
-int launch_fwd(const void* x, const void* gain, float eps, void* out, float* rstd, int64_t N, int H,
+int launch_fwd(const void* x, const float* gain, float eps, void* out, float* rstd, int64_t N, int H,
                bool vec, hipStream_t stream)
 {
     const dim3 grid(static_cast<unsigned>(N)), block(kNormThreads);
@@ -203,7 +201,7 @@ int launch_fwd(const void* x, const void* gain, float eps, void* out, float* rst
 }
 
 template <int DT>
-int launch_bwd(const void* x, const void* gain, float eps, const void* dout, void* dx, float* part,
+int launch_bwd(const void* x, const float* gain, float eps, const void* dout, void* dx, float* part,
                int64_t N, int H, bool vec, hipStream_t stream)
 {
     const unsigned groups = static_cast<unsigned>((N + kNormRowsPerGroup - 1) / kNormRowsPerGroup);
@@ -228,7 +226,7 @@ int launch_bwd(const void* x, const void* gain, float eps, const void* dout, voi
 
 }  // namespace
 
-int rmsnorm_fwd_enqueue(const void* x, const void* gain, float eps, void* out, float* rstd, int64_t N,
+int rmsnorm_fwd_enqueue(const void* x, const float* gain, float eps, void* out, float* rstd, int64_t N,
                         int32_t H, int32_t dtype, hipStream_t stream)
 {
     const bool vec = vec_ok(x, gain, out, H, dtype);
@@ -245,7 +243,7 @@ size_t rmsnorm_bwd_workspace(int64_t N, int32_t H)
     return groups * static_cast<size_t>(H) * sizeof(float);
 }
 
-int rmsnorm_bwd_enqueue(const void* x, const void* gain, float eps, const void* d_out, void* d_x,
+int rmsnorm_bwd_enqueue(const void* x, const float* gain, float eps, const void* d_out, void* d_x,
                         float* d_gain, int accumulate_gain, void* workspace, int64_t N, int32_t H,
                         int32_t dtype, hipStream_t stream)
 {
@@ -273,8 +271,9 @@ using namespace rlk;
 
 namespace {
 
-// Tokens whose normalised rows are held at a time by the fused entry points.
-constexpr int64_t kNormBlockTokens = 32768;
+// Tokens whose normalised rows are held at a time by the fused entry points (64 MiB of 16-bit rows
+// at H = 4096; the head runs within 2 % of its large-batch rate on 8192 tokens).
+constexpr int64_t kNormBlockTokens = 8192;
 
 inline size_t up256(size_t x) { return (x + 255) / 256 * 256; }
 inline size_t elt_bytes(int dtype) { return dtype == RLK_DTYPE_F32 ? 4 : 2; }
@@ -284,7 +283,7 @@ inline int64_t block_tokens(int64_t N) { return N < kNormBlockTokens ? N : kNorm
 
 extern "C" {
 
-int rlk_rmsnorm_fwd(const void* x, const void* gain, float eps, void* out, float* rstd, int64_t N,
+int rlk_rmsnorm_fwd(const void* x, const float* gain, float eps, void* out, float* rstd, int64_t N,
                     int32_t H, int32_t dtype, hipStream_t stream)
 {
     if (int rc = check_norm(x, gain, N, H, dtype)) return rc;
@@ -299,7 +298,7 @@ int rlk_rmsnorm_bwd_workspace_bytes(int64_t N, int32_t H, size_t* bytes)
     return 0;
 }
 
-int rlk_rmsnorm_bwd(const void* x, const void* gain, float eps, const void* d_out, void* d_x,
+int rlk_rmsnorm_bwd(const void* x, const float* gain, float eps, const void* d_out, void* d_x,
                     float* d_gain, void* workspace, size_t workspace_bytes, int64_t N, int32_t H,
                     int32_t dtype, hipStream_t stream)
 {
@@ -321,7 +320,7 @@ int rlk_linear_logp_rmsnorm_fwd_workspace_bytes(int64_t N, int32_t H, int64_t V,
     return 0;
 }
 
-int rlk_linear_logp_rmsnorm_fwd(const void* x, const void* gain, float eps, const void* weight,
+int rlk_linear_logp_rmsnorm_fwd(const void* x, const float* gain, float eps, const void* weight,
                                 const float* bias, const int64_t* targets, float* logp, float* lse,
                                 void* workspace, size_t workspace_bytes, int64_t N, int32_t H,
                                 int64_t V, int64_t vocab_start, int32_t dtype, float temperature,
@@ -360,12 +359,14 @@ int rlk_linear_logp_rmsnorm_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V,
     const int64_t nb = block_tokens(N);
     size_t bwd = 0;
     if (int rc = rlk_linear_logp_bwd_workspace_bytes(nb, H, V, dtype, dz_budget_bytes, &bwd)) return rc;
-    const size_t rows = up256(static_cast<size_t>(nb) * H * elt_bytes(dtype));
-    *bytes = 2 * rows + up256(rmsnorm_bwd_workspace(nb, H)) + up256(bwd);
+    // one block of normalised rows (+ 256 bytes so that it can be cut into two aligned halves, see
+    // rlk_linear_logp_rmsnorm_bwd); the gradient w.r.t. the normalised rows goes straight into d_x
+    const size_t rows = up256(static_cast<size_t>(nb) * H * elt_bytes(dtype)) + 256;
+    *bytes = rows + up256(rmsnorm_bwd_workspace(nb, H)) + up256(bwd);
     return 0;
 }
 
-int rlk_linear_logp_rmsnorm_bwd(const float* grad_logp, const void* x, const void* gain, float eps,
+int rlk_linear_logp_rmsnorm_bwd(const float* grad_logp, const void* x, const float* gain, float eps,
                                 const void* weight, const float* bias, const int64_t* targets,
                                 const float* lse, void* d_x, float* d_gain, float* d_weight,
                                 float* d_bias, void* workspace, size_t workspace_bytes,
@@ -381,31 +382,42 @@ int rlk_linear_logp_rmsnorm_bwd(const float* grad_logp, const void* x, const voi
     if (!workspace || workspace_bytes < need) return rlk_fail(RLK_ERR_ARG, "workspace too small");
     if (reinterpret_cast<uintptr_t>(workspace) & 255)
         return rlk_fail(RLK_ERR_ARG, "workspace must be 256-byte aligned");
-    const int64_t nb = block_tokens(N);
     const size_t es = elt_bytes(dtype);
-    const size_t rows = up256(static_cast<size_t>(nb) * H * es);
+    const int64_t nb_full = block_tokens(N);
+    const size_t rows = up256(static_cast<size_t>(nb_full) * H * es) + 256;
     char* ws = static_cast<char*>(workspace);
-    void* normed = ws;
-    void* d_normed = ws + rows;
-    void* gain_ws = ws + 2 * rows;
-    void* bwd_ws = ws + 2 * rows + up256(rmsnorm_bwd_workspace(nb, H));
-    const size_t bwd_bytes = need - (2 * rows + up256(rmsnorm_bwd_workspace(nb, H)));
+    void* gain_ws = ws + rows;
+    void* bwd_ws = ws + rows + up256(rmsnorm_bwd_workspace(nb_full, H));
+    const size_t bwd_bytes = need - (rows + up256(rmsnorm_bwd_workspace(nb_full, H)));
     const bool need_norm_bwd = d_x != nullptr || d_gain != nullptr;
+    // The head's gradient w.r.t. the normalised rows is written into the caller's d_x block and the
+    // norm backward then runs on it in place (a thread reads an element of d_out before it writes
+    // the same element of d_x, and the row's dot product is complete before the first write).
+    // Without d_x (only d_gain wanted) there is no such buffer: the block is halved and the second
+    // half of the row region holds that gradient.
+    const bool in_place = d_x != nullptr;
+    const int64_t nb = (in_place || !need_norm_bwd) ? nb_full : (nb_full + 1) / 2;
+    void* normed = ws;
+    void* d_half = ws + up256(static_cast<size_t>(nb) * H * es);
+    if (!in_place && need_norm_bwd) {
+        size_t half_need = 0;
+        if (int rc = rlk_linear_logp_bwd_workspace_bytes(nb, H, V, dtype, dz_budget_bytes, &half_need)) return rc;
+        if (half_need > bwd_bytes) return rlk_fail(RLK_ERR_ARG, "workspace too small");
+    }
     for (int64_t t0 = 0; t0 < N; t0 += nb) {
         const int64_t n = N - t0 < nb ? N - t0 : nb;
         const char* xb = static_cast<const char*>(x) + static_cast<size_t>(t0) * H * es;
+        void* dxb = d_x ? static_cast<char*>(d_x) + static_cast<size_t>(t0) * H * es : d_half;
         if (int rc = rmsnorm_fwd_enqueue(xb, gain, eps, normed, nullptr, n, H, dtype, stream)) return rc;
         // dW / db of the first block are written, those of later blocks added on top
         if (int rc = linear_logp_bwd_accumulating(grad_logp + t0, normed, weight, bias, targets + t0,
-                                                  lse + t0, need_norm_bwd ? d_normed : nullptr,
+                                                  lse + t0, need_norm_bwd ? dxb : nullptr,
                                                   d_weight, d_bias, bwd_ws, bwd_bytes, dz_budget_bytes,
                                                   n, H, V, vocab_start, dtype, temperature,
                                                   ignore_index, use_ignore, t0 > 0 ? 1 : 0, stream))
             return rc;
         if (need_norm_bwd) {
-            // d_x may be absent (only d_gain wanted): the rows of d_normed are then overwritten in place
-            void* dxb = d_x ? static_cast<char*>(d_x) + static_cast<size_t>(t0) * H * es : d_normed;
-            if (int rc = rmsnorm_bwd_enqueue(xb, gain, eps, d_normed, dxb, d_gain, t0 > 0 ? 1 : 0, gain_ws,
+            if (int rc = rmsnorm_bwd_enqueue(xb, gain, eps, dxb, dxb, d_gain, t0 > 0 ? 1 : 0, gain_ws,
                                              n, H, dtype, stream))
                 return rc;
         }

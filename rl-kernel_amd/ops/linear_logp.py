@@ -210,6 +210,7 @@ def fused_norm_linear_logp_forward(
     if n == 0:
         return logp, lse, err
     _warn_if_wide_path(x_2d, weight)
+    gain = _aligned_contiguous(gain.detach().to(torch.float32))  # the library takes an fp32 gain
     need = _native.ctypes.c_size_t(0)
     dt = _DTYPES[x_2d.dtype]
     _native.check(lib.rlk_linear_logp_rmsnorm_fwd_workspace_bytes(n, h, v, dt, _native.ctypes.byref(need)),
@@ -251,6 +252,7 @@ def fused_norm_linear_logp_backward(
     v = weight.size(0)
     dev = x_2d.device
     dt = _DTYPES[x_2d.dtype]
+    gain = _aligned_contiguous(gain.detach().to(torch.float32))  # the library takes an fp32 gain
     g = grad_logp.reshape(-1).to(torch.float32).contiguous()
     d_x = torch.empty_like(x_2d) if need_x else None
     d_gain = torch.empty(h, device=dev, dtype=torch.float32) if need_gain else None
@@ -421,7 +423,7 @@ class _FusedNormLinearLogpFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, gain, weight, bias, target_ids, eps, temperature, ignore_index, check_targets):
         x_2d = _aligned_contiguous(x.reshape(-1, x.size(-1)))
-        g = _aligned_contiguous(gain.to(x.dtype))
+        g = _aligned_contiguous(gain.detach().to(torch.float32))  # the reference multiplies by weight.float()
         w = _aligned_contiguous(weight)
         target_1d = target_ids.reshape(-1).to(device=x_2d.device, dtype=torch.long).contiguous()
         logp, lse, err = fused_norm_linear_logp_forward(

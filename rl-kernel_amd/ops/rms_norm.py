@@ -17,11 +17,12 @@ from .linear_logp import _DTYPES, _aligned_contiguous, _ptr, _stream
 
 @_native.on_tensor_device
 def rmsnorm_forward(x_2d: torch.Tensor, gain: torch.Tensor, eps: float) -> torch.Tensor:
-    """Raw launch: normalised rows in the dtype of ``x_2d`` ([N, H] contiguous, gain [H] same dtype)."""
+    """Raw launch: normalised rows in the dtype of ``x_2d`` ([N, H] contiguous, gain [H] float32)."""
     out = torch.empty_like(x_2d)
     n, h = x_2d.shape
     if n == 0:
         return out
+    gain = _aligned_contiguous(gain.detach().to(torch.float32))
     rc = _native.load().rlk_rmsnorm_fwd(_ptr(x_2d), _ptr(gain), float(eps), _ptr(out), None, n, h,
                                         _DTYPES[x_2d.dtype], _stream(x_2d.device))
     _native.check(rc, "rlk_rmsnorm_fwd")
@@ -37,6 +38,7 @@ def rmsnorm_backward(x_2d: torch.Tensor, gain: torch.Tensor, eps: float, d_out: 
     d_gain = torch.zeros(h, device=x_2d.device, dtype=torch.float32)
     if n == 0:
         return d_x, d_gain
+    gain = _aligned_contiguous(gain.detach().to(torch.float32))
     need = _native.ctypes.c_size_t(0)
     _native.check(lib.rlk_rmsnorm_bwd_workspace_bytes(n, h, _native.ctypes.byref(need)),
                   "rmsnorm backward workspace query")
@@ -51,7 +53,7 @@ class _RMSNormFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, eps):
         x_2d = _aligned_contiguous(x.reshape(-1, x.size(-1)))
-        gain = _aligned_contiguous(weight.to(x.dtype))
+        gain = _aligned_contiguous(weight.detach().to(torch.float32))  # the reference multiplies by weight.float()
         ctx.save_for_backward(x_2d, gain)
         ctx.eps = eps
         ctx.x_shape = x.shape

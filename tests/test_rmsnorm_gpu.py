@@ -123,7 +123,7 @@ def test_norm_fused_linear_logp_matches_oracle_and_the_unfused_kernels(dev, lead
 
 
 def test_norm_fused_path_walks_several_token_blocks(dev):
-    """More than 32768 tokens: the normalised rows exist one block at a time, dW and d_gain are added
+    """More than 8192 tokens: the normalised rows exist one block at a time, dW and d_gain are added
     up across the blocks; checked against the unfused kernels (bitwise forward, gradients within the
     rounding of another summation order) and, on sampled rows, against the oracle."""
     from rl_kernel_amd import _native
@@ -131,7 +131,7 @@ def test_norm_fused_path_walks_several_token_blocks(dev):
     from rl_kernel_amd.ops.rms_norm import rmsnorm_backward, rmsnorm_forward
     import ctypes
 
-    n, h, v = 70000, 512, 4096
+    n, h, v, blk = 20000, 512, 4096, 8192
     g = torch.Generator(device=dev).manual_seed(8)
     x = (torch.randn(n, h, device=dev, generator=g) * 2).to(torch.bfloat16)
     gain = (1.0 + 0.2 * torch.randn(h, device=dev, generator=g)).to(torch.bfloat16)
@@ -142,13 +142,13 @@ def test_norm_fused_path_walks_several_token_blocks(dev):
     assert int(err.item()) == 0
     d_x, d_g, d_w, _ = LL.fused_norm_linear_logp_backward(up, x, gain, w, tgt, lse, eps=1e-5,
                                                           temperature=0.9)
-    # the unfused kernels on the same blocks of 32768 tokens (the launch plan, hence the summation
+    # the unfused kernels on the same blocks of 8192 tokens (the launch plan, hence the summation
     # order inside a row, is a function of the token count of a call)
     hn = rmsnorm_forward(x, gain, 1e-5)
     dw_u = torch.zeros_like(d_w)
     dg_u = torch.zeros_like(d_g)
-    for t0 in range(0, n, 32768):
-        sl = slice(t0, min(n, t0 + 32768))
+    for t0 in range(0, n, blk):
+        sl = slice(t0, min(n, t0 + blk))
         logp_u, lse_u, _ = LL.fused_linear_logp_forward(hn[sl], w, tgt[sl], temperature=0.9)
         assert torch.equal(logp[sl], logp_u) and torch.equal(lse[sl], lse_u)
         dh_b, dw_b, _ = LL.fused_linear_logp_backward(up[sl], hn[sl], w, tgt[sl], lse[sl], temperature=0.9)
@@ -157,7 +157,7 @@ def test_norm_fused_path_walks_several_token_blocks(dev):
         dw_u += dw_b
         dg_u += dg_b
     assert rel(d_w, dw_u) < 1e-5 and rel(d_g, dg_u) < 1e-5
-    rows = torch.tensor([0, 32767, 32768, 65535, 65536, n - 1])
+    rows = torch.tensor([0, blk - 1, blk, 2 * blk - 1, 2 * blk, n - 1])
     want = O.linear_logp(O.rms_norm(x[rows].cpu(), gain.cpu(), eps=1e-5), w.cpu(), tgt[rows].cpu(),
                          temperature=0.9)
     assert (logp[rows].cpu() - want).abs().max().item() < 1e-3
@@ -169,4 +169,53 @@ def test_norm_fused_path_walks_several_token_blocks(dev):
         assert lib.rlk_linear_logp_rmsnorm_bwd_workspace_bytes(tokens, 4096, 128256, 0, 0,
                                                                ctypes.byref(need)) == 0
         sizes.append(need.value)
-    assert sizes[0] == sizes[1] == sizes[2] and sizes[0] < (1 << 30)
+    assert sizes[0] == sizes[1] == sizes[2] and sizes[0] <= (1 << 29)   # at most 0.5 GiB at the Llama head
+    need = ctypes.c_size_t(0)
+    assert lib.rlk_linear_logp_rmsnorm_fwd_workspace_bytes(32768, 4096, 128256, 0, ctypes.byref(need)) == 0
+    assert need.value <= (1 << 27)
+    # only d_gain wanted: no d_x buffer to run the norm backward in, the blocks are halved instead
+    _, d_g2, _, _ = LL.fused_norm_linear_logp_backward(up, x, gain, w, tgt, lse, eps=1e-5, temperature=0.9,
+                                                      need_x=False, need_weight=False)
+    assert rel(d_g2, dg_u) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fp32_gain_over_16_bit_activations_is_not_rounded(dev, dtype):
+    """The reference multiplies by weight.float() (rl_engine/kernels/ops/pytorch/norm/rms_norm.py:66-70):
+    an fp32 gain over 16-bit activations must enter the product unrounded.  The gain here is chosen
+    so that rounding it to the activation dtype first would move many outputs by one unit in the
+    last place: the result must equal the oracle's (fp32 gain) wherever the two differ."""
+    from rl_kernel_amd.ops.linear_logp import RocmFusedLinearLogpOp
+    from rl_kernel_amd.ops.rms_norm import RocmRMSNormOp
+
+    g = torch.Generator().manual_seed(77)
+    n, h, v = 192, 256, 700
+    x = (torch.randn(n, h, generator=g) * 2.0).to(dtype)
+    gain = 1.0 + 0.37 * torch.rand(h, generator=g) + 1.0 / 1024.0 / 3.0   # fp32, off the 16-bit grids
+    assert not torch.equal(gain.to(dtype).float(), gain)
+    want = O.rms_norm(x, gain)
+    rounded_first = O.rms_norm(x, gain.to(dtype))
+    assert (want != rounded_first).float().mean().item() > 0.02      # the case does discriminate
+    got = RocmRMSNormOp()(x.to(dev), gain.to(dev)).cpu()
+    # same fp32 expression as the oracle: at most one unit in the last place apart, and strictly
+    # closer to the unrounded-gain result than to the rounded-gain one
+    assert torch.allclose(got.float(), want.float(), rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10,
+                          atol=1e-6)
+    assert (got != want).float().mean().item() < 0.25 * (rounded_first != want).float().mean().item() + 1e-3
+
+    go = torch.randn(n, h, generator=g).to(dtype)
+    xd, gd = x.to(dev).requires_grad_(True), gain.to(dev).requires_grad_(True)
+    RocmRMSNormOp()(xd, gd).backward(go.to(dev))
+    d_x, d_w = O.rms_norm_backward(go, x, gain)
+    assert gd.grad.dtype == torch.float32
+    assert rel(xd.grad, d_x) < 1e-2 and rel(gd.grad, d_w) < 1e-4
+
+    # the norm inside the head takes the fp32 gain too: same bits as norm op -> head op
+    w = (torch.randn(v, h, generator=g) * 0.1).to(dtype)
+    tgt = torch.randint(0, v, (n,), generator=g)
+    op = RocmFusedLinearLogpOp()
+    fused = op(x.to(dev), w.to(dev), tgt.to(dev), norm_weight=gain.to(dev))
+    unfused = op(RocmRMSNormOp()(x.to(dev), gain.to(dev)), w.to(dev), tgt.to(dev))
+    assert torch.equal(fused, unfused)
+    ref = O.linear_logp(O.rms_norm(x, gain), w, tgt)
+    assert (fused.cpu() - ref).abs().max().item() < 1e-3
