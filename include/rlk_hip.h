@@ -111,8 +111,10 @@ int rlk_linear_logp_fwd_static(const void* hidden, const void* weight, const flo
  * for the KL term (rl_engine/executors/deepspeed_trainer.py:146-167); the logits-fed counterpart
  * in the reference is the single program that scans both logit rows
  * (rl_engine/kernels/ops/triton/loss/ratio_kl.py:46-60).  Only the policy head is strict about
- * targets; both heads must have a bias or neither.  Workspace: twice the single-head size
- * (rlk_linear_logp_fwd_pair_workspace_bytes). */
+ * targets; both heads must have a bias or neither, and both weights must be 16-byte aligned or
+ * neither (the two heads share one launch, hence one kind of kernel; a mixed pair is answered with
+ * RLK_ERR_UNSUPPORTED rather than by moving the aligned head to the fp32 kernels).  Workspace:
+ * twice the single-head size (rlk_linear_logp_fwd_pair_workspace_bytes). */
 int rlk_linear_logp_fwd_pair_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                              size_t* bytes);
 

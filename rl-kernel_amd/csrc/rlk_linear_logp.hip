@@ -1603,8 +1603,15 @@ int fwd_enqueue(const void* hidden, const void* weight, const float* bias, const
     if (!hidden || !weight || !targets || !logp || !lse) return rlk_fail(RLK_ERR_ARG, "null pointer");
     if (strict_targets && !err_flag)
         return rlk_fail(RLK_ERR_ARG, "strict_targets needs an err_flag to report through");
-    const bool mfma = use_mfma(hidden, weight, H, dtype) &&
-                      (second == nullptr || use_mfma(hidden, second->weight, H, dtype));
+    const bool mfma = use_mfma(hidden, weight, H, dtype);
+    // Both heads of a pair run through one launch, so they must take the same kind of kernel:
+    // otherwise the policy head's results would depend on the reference head's alignment and no
+    // longer equal the single-head call bit for bit.
+    if (second != nullptr && use_mfma(hidden, second->weight, H, dtype) != mfma)
+        return rlk_fail(RLK_ERR_UNSUPPORTED,
+                        "rlk_linear_logp_fwd_pair: weight and ref_weight must both start on a 16-byte "
+                        "boundary or neither (one would run on the 16-bit MFMA tiles, the other on the "
+                        "fp32 matrix-core kernels); call rlk_linear_logp_fwd once per head instead");
     size_t need = 0;
     rlk_linear_logp_fwd_workspace_bytes(N, H, V, dtype, &need);
     if (second != nullptr) need *= 2;

@@ -148,3 +148,40 @@ def test_logits_pair_scan_equals_two_scans(dev, dtype):
         assert torch.equal(lses[0], lses[2]) and torch.equal(lses[1], lses[3])
     want = O.logp_from_logits(b.cpu(), ids.cpu())
     assert (outs[1][torch.tensor([0, 5, 76, 40])].cpu() - want[torch.tensor([0, 5, 76, 40])]).abs().max() < 2e-3
+
+
+def test_pair_with_heads_of_different_alignment_is_refused_not_rerouted(dev):
+    """Raw C ABI: a 16-byte aligned policy head with a misaligned reference head would put both on
+    the fp32 matrix-core kernels and change the policy head's bits; the call is answered with
+    RLK_ERR_UNSUPPORTED and enqueues nothing.  (The Python op re-aligns its inputs.)"""
+    import ctypes
+
+    from rl_kernel_amd import _native
+
+    lib = _native.load()
+    n, h, v = 64, 64, 512
+    hidden = torch.randn(n, h, device=dev).to(torch.bfloat16)
+    w = (torch.randn(v, h, device=dev) * 0.1).to(torch.bfloat16)
+    store = torch.empty(v * h + 8, device=dev, dtype=torch.bfloat16)
+    w_ref = store[1:1 + v * h].view(v, h)            # starts 2 bytes past a 16-byte boundary
+    w_ref.copy_(w)
+    assert w.data_ptr() % 16 == 0 and w_ref.data_ptr() % 16 != 0
+    tgt = torch.randint(0, v, (n,), device=dev)
+    outs = [torch.full((n,), 5.0, device=dev) for _ in range(4)]
+    err = torch.zeros(1, device=dev, dtype=torch.int32)
+    need = ctypes.c_size_t(0)
+    assert lib.rlk_linear_logp_fwd_pair_workspace_bytes(n, h, v, 0, ctypes.byref(need)) == 0
+    ws = torch.empty(max(need.value, 16), device=dev, dtype=torch.uint8)
+    rc = lib.rlk_linear_logp_fwd_pair(hidden.data_ptr(), w.data_ptr(), w_ref.data_ptr(), None, None,
+                                      tgt.data_ptr(), *[o.data_ptr() for o in outs], ws.data_ptr(), ws.numel(),
+                                      n, h, v, 0, 0, 1.0, 0, 0, 1, err.data_ptr(),
+                                      torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == -2 and b"16-byte" in lib.rlk_last_error()
+    assert all(torch.equal(o, torch.full((n,), 5.0, device=dev)) for o in outs)   # nothing was written
+    # the op re-aligns what it is given: same call through Python works and matches the single heads
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    a = LL.fused_linear_logp_forward_pair(hidden, w, LL._aligned_contiguous(w_ref), tgt)
+    b = LL.fused_linear_logp_forward(hidden, w, tgt)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[2], b[0])

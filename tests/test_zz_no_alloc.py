@@ -38,11 +38,24 @@ def _call_pair(lib, n, h, v, dtype, seed, temperature, with_ignore, with_bias):
                   stream)
         bias_p = None if bias is None else bias.data_ptr()
         if static:
+            def call_static():
+                return lib.rlk_linear_logp_fwd_static(hidden.data_ptr(), weight.data_ptr(), bias_p,
+                                                      targets.data_ptr(), logp.data_ptr(),
+                                                      lse.data_ptr(), *common)
+
+            # one call to get the per-device set-up out of the way (symbol address, kernel
+            # attributes, code object load), then the measured one: the driver's count of free
+            # device memory sees a hipMalloc inside the library, which torch's allocator
+            # statistics would not
+            assert call_static() == 0, lib.rlk_last_error()
+            torch.cuda.synchronize()
             before = torch.cuda.memory_allocated(dev)
-            rc = lib.rlk_linear_logp_fwd_static(hidden.data_ptr(), weight.data_ptr(), bias_p,
-                                                targets.data_ptr(), logp.data_ptr(),
-                                                lse.data_ptr(), *common)
+            free_before, _ = torch.cuda.mem_get_info(dev)
+            rc = call_static()
+            torch.cuda.synchronize()
+            free_after, _ = torch.cuda.mem_get_info(dev)
             assert torch.cuda.memory_allocated(dev) == before
+            assert free_after == free_before, "the static entry point changed the device's free memory"
         else:
             rc = lib.rlk_linear_logp_fwd(hidden.data_ptr(), weight.data_ptr(), bias_p,
                                          targets.data_ptr(), logp.data_ptr(), lse.data_ptr(),
