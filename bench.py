@@ -452,7 +452,7 @@ def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False
 
     if registry_op and do_bwd and not grpo:
         res["through_registry_op"] = bench_registry_op(torch, hidden, weight, targets, grad, temp, ign,
-                                                       max(2, steps // 4))
+                                                       max(3, steps // 2))
     return res
 
 

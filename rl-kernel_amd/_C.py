@@ -9,12 +9,11 @@ below.  ``COMPILED`` says which one is bound."""
 
 from __future__ import annotations
 
-import importlib.util
-import os
 from typing import List, Optional
 
 import torch
 
+from . import _compiled
 from .ops.linear_logp import _aligned_contiguous, fused_linear_logp_forward
 from .ops.logp import logp_from_logits
 
@@ -80,19 +79,9 @@ fused_linear_logp_sm90 = fused_linear_logp
 
 
 
-def _load_compiled():
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "_rlk_C.so")
-    if not os.path.exists(path):
-        return None
-    spec = importlib.util.spec_from_file_location("_rlk_C", path)
-    module = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(module)
-    return module
-
-
 _PYTHON_ROUTE = {name: obj for name, obj in list(globals().items())
                  if name.startswith("fused_") and callable(obj)}
-compiled_module = _load_compiled()
+compiled_module = _compiled.module()
 COMPILED = compiled_module is not None
 if COMPILED:
     for _name in _PYTHON_ROUTE:

@@ -73,6 +73,113 @@ std::vector<at::Tensor> fused_linear_logp(at::Tensor hidden, at::Tensor weight, 
     return {logp, lse};
 }
 
+// Forward with the keyword extensions of the op classes (temperature, ignore-index, strictness):
+// [logp, lse, err_flag]; err_flag (int32[1], device) is non-zero when strict_targets and a
+// non-ignored target lies outside the shard.  Does not synchronise.
+std::vector<at::Tensor> fused_linear_logp_forward_ex(at::Tensor hidden, at::Tensor weight, at::Tensor target,
+                                                     c10::optional<at::Tensor> bias, double temperature,
+                                                     c10::optional<int64_t> ignore_index, int64_t vocab_start,
+                                                     bool strict_targets)
+{
+    TORCH_CHECK(hidden.dim() == 2 && weight.dim() == 2, "hidden and weight must be 2D tensors");
+    TORCH_CHECK(hidden.is_cuda() && weight.is_cuda(), "hidden and weight must be CUDA tensors");
+    const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(hidden.device());
+    TORCH_CHECK(weight.size(1) == hidden.size(1), "hidden/weight hidden-dim mismatch");
+    TORCH_CHECK(target.numel() == hidden.size(0), "target must have one id per token");
+    TORCH_CHECK(weight.scalar_type() == hidden.scalar_type(), "hidden and weight must share a dtype");
+    TORCH_CHECK(hidden.is_contiguous() && weight.is_contiguous(), "hidden and weight must be contiguous");
+    TORCH_CHECK(target.scalar_type() == at::kLong && target.is_contiguous() && target.is_cuda(),
+                "target must be a contiguous int64 CUDA tensor");
+    const int dt = dtype_id(hidden.scalar_type());
+    TORCH_CHECK(dt == RLK_DTYPE_BF16 || dt == RLK_DTYPE_F16 || dt == RLK_DTYPE_F32,
+                "hidden dtype must be bfloat16, float16 or float32");
+    const int64_t n = hidden.size(0), v = weight.size(0);
+    const int32_t hd = static_cast<int32_t>(hidden.size(1));
+    auto f32 = hidden.options().dtype(at::kFloat);
+    auto logp = at::empty({n}, f32), lse = at::empty({n}, f32);
+    auto err = at::zeros({1}, hidden.options().dtype(at::kInt));
+    if (n == 0) return {logp, lse, err};
+    size_t ws_bytes = 0;
+    TORCH_CHECK(rlk_linear_logp_fwd_workspace_bytes(n, hd, v, dt, &ws_bytes) == 0, rlk_last_error());
+    auto ws = at::empty({static_cast<int64_t>(ws_bytes < 16 ? 16 : ws_bytes)}, hidden.options().dtype(at::kByte));
+    at::Tensor bias_f;
+    const float* bias_p = nullptr;
+    if (bias.has_value() && bias->defined()) {
+        TORCH_CHECK(bias->numel() == v, "bias must have one value per vocab row");
+        bias_f = bias->detach().to(hidden.device(), at::kFloat).contiguous();
+        bias_p = bias_f.data_ptr<float>();
+    }
+    const int rc = rlk_linear_logp_fwd(hidden.data_ptr(), weight.data_ptr(), bias_p, target.data_ptr<int64_t>(),
+                                       logp.data_ptr<float>(), lse.data_ptr<float>(), ws.data_ptr(),
+                                       static_cast<size_t>(ws.numel()), n, hd, v, vocab_start, dt,
+                                       static_cast<float>(temperature), ignore_index.value_or(0),
+                                       ignore_index.has_value() ? 1 : 0, strict_targets ? 1 : 0,
+                                       err.data_ptr<int32_t>(), current_stream(hidden));
+    TORCH_CHECK(rc != RLK_ERR_ARG, "rlk_linear_logp_fwd: ", rlk_last_error());
+    TORCH_CHECK(rc == 0, "rlk_linear_logp_fwd: ", rlk_last_error());
+    return {logp, lse, err};
+}
+
+// Backward: [d_hidden (input dtype), d_weight (f32), d_bias (f32)], an undefined tensor for every
+// gradient that is not wanted.  weight_grad_out / bias_grad_out: caller-owned fp32 buffers that
+// receive (accumulate: are added) the gradients and are what the call returns in their place.
+std::vector<at::Tensor> fused_linear_logp_backward(at::Tensor grad_logp, at::Tensor hidden, at::Tensor weight,
+                                                   at::Tensor target, at::Tensor lse,
+                                                   c10::optional<at::Tensor> bias, double temperature,
+                                                   c10::optional<int64_t> ignore_index, int64_t vocab_start,
+                                                   bool need_hidden, bool need_weight, bool need_bias,
+                                                   int64_t dz_budget_bytes,
+                                                   c10::optional<at::Tensor> weight_grad_out,
+                                                   c10::optional<at::Tensor> bias_grad_out, bool accumulate)
+{
+    TORCH_CHECK(hidden.dim() == 2 && weight.dim() == 2, "hidden and weight must be 2D tensors");
+    TORCH_CHECK(hidden.is_cuda() && weight.is_cuda(), "hidden and weight must be CUDA tensors");
+    const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(hidden.device());
+    TORCH_CHECK(hidden.is_contiguous() && weight.is_contiguous(), "hidden and weight must be contiguous");
+    TORCH_CHECK(target.scalar_type() == at::kLong && target.is_contiguous() && target.is_cuda(),
+                "target must be a contiguous int64 CUDA tensor");
+    TORCH_CHECK(lse.scalar_type() == at::kFloat && lse.is_contiguous(), "lse must be contiguous float32");
+    const int dt = dtype_id(hidden.scalar_type());
+    TORCH_CHECK(dt == RLK_DTYPE_BF16 || dt == RLK_DTYPE_F16 || dt == RLK_DTYPE_F32,
+                "hidden dtype must be bfloat16, float16 or float32");
+    const int64_t n = hidden.size(0), v = weight.size(0);
+    const int32_t hd = static_cast<int32_t>(hidden.size(1));
+    auto g = grad_logp.reshape({-1}).to(at::kFloat).contiguous();
+    TORCH_CHECK(g.numel() == n, "grad_logp must have one value per token");
+    auto f32 = hidden.options().dtype(at::kFloat);
+    const bool has_bias = bias.has_value() && bias->defined();
+    const bool want_bias = has_bias && need_bias;
+    at::Tensor d_hidden, d_weight, d_bias, bias_f;
+    if (need_hidden) d_hidden = at::empty_like(hidden);
+    if (need_weight) d_weight = weight_grad_out.has_value() && weight_grad_out->defined() ? *weight_grad_out
+                                                                                          : at::empty({v, hd}, f32);
+    if (want_bias) d_bias = bias_grad_out.has_value() && bias_grad_out->defined() ? *bias_grad_out : at::empty({v}, f32);
+    if (d_weight.defined())
+        TORCH_CHECK(d_weight.scalar_type() == at::kFloat && d_weight.is_contiguous() && d_weight.numel() == v * hd,
+                    "weight_grad_out must be contiguous float32 [V, H]");
+    if (d_bias.defined())
+        TORCH_CHECK(d_bias.scalar_type() == at::kFloat && d_bias.is_contiguous() && d_bias.numel() == v,
+                    "bias_grad_out must be contiguous float32 [V]");
+    const float* bias_p = nullptr;
+    if (has_bias) {
+        bias_f = bias->detach().to(hidden.device(), at::kFloat).contiguous();
+        bias_p = bias_f.data_ptr<float>();
+    }
+    size_t ws_bytes = 0;
+    TORCH_CHECK(rlk_linear_logp_bwd_workspace_bytes(n, hd, v, dt, static_cast<size_t>(dz_budget_bytes), &ws_bytes) == 0,
+                rlk_last_error());
+    auto ws = at::empty({static_cast<int64_t>(ws_bytes)}, hidden.options().dtype(at::kByte));
+    const int rc = rlk_linear_logp_bwd_accum(
+        g.data_ptr<float>(), hidden.data_ptr(), weight.data_ptr(), bias_p, target.data_ptr<int64_t>(),
+        lse.data_ptr<float>(), d_hidden.defined() ? d_hidden.data_ptr() : nullptr,
+        d_weight.defined() ? d_weight.data_ptr<float>() : nullptr,
+        d_bias.defined() ? d_bias.data_ptr<float>() : nullptr, ws.data_ptr(), static_cast<size_t>(ws.numel()),
+        static_cast<size_t>(dz_budget_bytes), n, hd, v, vocab_start, dt, static_cast<float>(temperature),
+        ignore_index.value_or(0), ignore_index.has_value() ? 1 : 0, accumulate ? 1 : 0, current_stream(hidden));
+    TORCH_CHECK(rc == 0, "rlk_linear_logp_bwd_accum: ", rlk_last_error());
+    return {d_hidden, d_weight, d_bias};
+}
+
 // Selected-token log-prob of materialised logits into `output` (all rows, or only row_indices).
 at::Tensor scan_into(const at::Tensor& logits, const at::Tensor& token_ids,
                      const c10::optional<at::Tensor>& row_indices, at::Tensor output)
@@ -154,6 +261,21 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("fused_linear_logp_sm90", &fused_linear_logp, "Fused linear log-prob -> [logp, lse]",
           pybind11::arg("hidden"), pybind11::arg("weight"), pybind11::arg("target"),
           pybind11::arg("bias") = pybind11::none());
+    m.def("fused_linear_logp_forward_ex", &fused_linear_logp_forward_ex,
+          "Fused linear log-prob with temperature / ignore-index -> [logp, lse, err_flag]",
+          pybind11::arg("hidden"), pybind11::arg("weight"), pybind11::arg("target"),
+          pybind11::arg("bias") = pybind11::none(), pybind11::arg("temperature") = 1.0,
+          pybind11::arg("ignore_index") = pybind11::none(), pybind11::arg("vocab_start") = 0,
+          pybind11::arg("strict_targets") = true);
+    m.def("fused_linear_logp_backward", &fused_linear_logp_backward,
+          "Backward of the fused linear log-prob -> [d_hidden, d_weight (f32), d_bias (f32)]",
+          pybind11::arg("grad_logp"), pybind11::arg("hidden"), pybind11::arg("weight"),
+          pybind11::arg("target"), pybind11::arg("lse"), pybind11::arg("bias") = pybind11::none(),
+          pybind11::arg("temperature") = 1.0, pybind11::arg("ignore_index") = pybind11::none(),
+          pybind11::arg("vocab_start") = 0, pybind11::arg("need_hidden") = true,
+          pybind11::arg("need_weight") = true, pybind11::arg("need_bias") = true,
+          pybind11::arg("dz_budget_bytes") = 0, pybind11::arg("weight_grad_out") = pybind11::none(),
+          pybind11::arg("bias_grad_out") = pybind11::none(), pybind11::arg("accumulate") = false);
     m.def("fused_logp_forward_out", &fused_logp_forward_out, "Fused logp out");
     m.def("fused_logp_forward_fp32", &fused_logp_forward_fp32, "Fused logp fp32");
     m.def("fused_logp_forward_indexed_out", &fused_logp_forward_indexed_out, "Fused logp indexed out");

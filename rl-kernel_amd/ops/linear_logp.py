@@ -14,7 +14,7 @@ from typing import Any, Optional
 
 import torch
 
-from .. import _native
+from .. import _compiled, _native
 from ..platform import logger
 
 _DTYPES = {torch.bfloat16: _native.DTYPE_BF16, torch.float16: _native.DTYPE_F16,
@@ -119,6 +119,15 @@ def fused_linear_logp_forward(
     n, h = hidden_2d.shape
     v = weight.size(0)
     dev = hidden_2d.device
+    compiled = _compiled.module()
+    if compiled is not None and n > 0 and hidden_2d.is_contiguous() and weight.is_contiguous() \
+            and target_1d.dtype == torch.long and target_1d.is_contiguous():
+        # same C ABI through the compiled binding: no per-argument ctypes marshalling
+        _warn_if_wide_path(hidden_2d, weight)
+        logp, lse, err = compiled.fused_linear_logp_forward_ex(
+            hidden_2d, weight, target_1d, bias, float(temperature), ignore_index, int(vocab_start),
+            bool(strict_targets))
+        return logp, lse, err
     logp = torch.empty(n, device=dev, dtype=torch.float32)
     lse = torch.empty(n, device=dev, dtype=torch.float32)
     err = torch.zeros(1, device=dev, dtype=torch.int32)
@@ -319,6 +328,15 @@ def fused_linear_logp_backward(
         _check_grad_buffer("bias_grad_out", bias_grad_out, (v,), dev)
     if accumulate and ((need_weight and weight_grad_out is None) or (want_bias and bias_grad_out is None)):
         raise ValueError("accumulate=True needs the buffers to add to (weight_grad_out / bias_grad_out)")
+    compiled = _compiled.module()
+    if compiled is not None and hidden_2d.is_contiguous() and weight.is_contiguous() \
+            and target_1d.dtype == torch.long and target_1d.is_contiguous() \
+            and lse.dtype == torch.float32 and lse.is_contiguous():
+        d_hidden, d_weight, d_bias = compiled.fused_linear_logp_backward(
+            grad_logp, hidden_2d, weight, target_1d, lse, bias, float(temperature), ignore_index,
+            int(vocab_start), bool(need_hidden), bool(need_weight), bool(want_bias),
+            int(dz_budget_bytes), weight_grad_out, bias_grad_out, bool(accumulate))
+        return d_hidden, d_weight, d_bias
     d_weight = None
     if need_weight:
         d_weight = weight_grad_out if weight_grad_out is not None else \
