@@ -102,24 +102,22 @@ def kernel_source_sha16() -> str:
 
 
 def make_inputs(torch, cfg, device, seed=1002):
-    gen = torch.Generator(device=device).manual_seed(seed)
+    """hidden ~ N(0,1), weight ~ N(0, 0.02^2), targets uniform (a Bernoulli(ignore_frac) share set
+    to -100), upstream gradient ~ N(0,1), from the counter-based generator: every value is a function
+    of (seed, tensor id, element index) in integer arithmetic, so the inputs do not depend on the
+    device or on the torch / rocRAND build (tensor ids: 0 hidden, 1 weight, 2 targets, 3 ignored
+    positions, 4 upstream gradient)."""
+    from rl_kernel_amd import synthetic as S
+
     dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float16
     n, h, v = cfg["tokens"], cfg["hidden"], cfg["vocab"]
-    hidden = torch.empty(n, h, device=device, dtype=dt)
-    step = 16384  # generate in slabs to bound the fp32 temporary
-    for n0 in range(0, n, step):
-        n1 = min(n, n0 + step)
-        hidden[n0:n1] = torch.randn(n1 - n0, h, device=device, dtype=torch.float32, generator=gen).to(dt)
-    weight = torch.empty(v, h, device=device, dtype=dt)
-    for v0 in range(0, v, step):
-        v1 = min(v, v0 + step)
-        weight[v0:v1] = (torch.randn(v1 - v0, h, device=device, dtype=torch.float32,
-                                     generator=gen) * 0.02).to(dt)
-    targets = torch.randint(0, v, (n,), device=device, generator=gen)
+    hidden = S.normal(seed, 0, (n, h), dtype=dt, device=device)
+    weight = S.normal(seed, 1, (v, h), std=0.02, dtype=dt, device=device)
+    targets = S.randint(seed, 2, (n,), v, device=device)
     if cfg["ignore_frac"] > 0:
-        drop = torch.rand(n, device=device, generator=gen) < cfg["ignore_frac"]
+        drop = S.bernoulli(seed, 3, (n,), cfg["ignore_frac"], device=device)
         targets = torch.where(drop, torch.full_like(targets, -100), targets)
-    grad = torch.randn(n, device=device, dtype=torch.float32, generator=gen)
+    grad = S.normal(seed, 4, (n,), device=device)
     return hidden, weight, targets, grad
 
 
@@ -736,7 +734,10 @@ def main() -> int:
     if args.dtype:
         cfg["dtype"] = args.dtype
     common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
-              "scaling": "weak", "vs_baseline": None, "data": "synthetic", "seed": 1002}
+              "scaling": "weak", "vs_baseline": None, "data": "synthetic", "seed": 1002,
+              "input_generator": "counter-based: splitmix64(seed, tensor id, index) -> Irwin-Hall normal / "
+                                 "uniform index in integer arithmetic (rl-kernel_amd/synthetic.py), the same "
+                                 "bits on CPU and GPU"}
 
     if args.calibrate_copy:
         src = torch.ones(1 << 28, device=dev, dtype=torch.float32)   # 1 GiB read + 1 GiB written
