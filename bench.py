@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "ed990790b256785d",
-    "measured_at_commit": "43286d2",
+    "kernel_source_sha16": "89e08cbb44fc092a",
+    "measured_at_commit": "04fb7f0",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 52009413181,
-        "linear_logp_dz_kernel": 1963094859,
-        "linear_logp_dh_kernel": 1893046182,
-        "linear_logp_dw_kernel": 2162991501,
+        "linear_logp_fwd_kernel": 56960450635,
+        "linear_logp_dz_kernel": 1953398134,
+        "linear_logp_dh_kernel": 1836843252,
+        "linear_logp_dw_kernel": 2110189437,
     },
 }
 
