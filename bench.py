@@ -390,6 +390,10 @@ def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False
             "active_tokens": int(mask.sum().item()),
         }
 
+    if grpo and kernel_timing:
+        res["skip_masked"] = bench_skip_masked(torch, hidden, weight, targets, mask, old, ref, rewards,
+                                               grpo, temp, max(3, steps // 2))
+
     # per-kernel launch times by HIP events: the forward on its own; the three backward kernels
     # from backward calls with one gradient switched off (dZ+dH, dZ+dW, all three), by difference
     if not kernel_timing:
@@ -452,6 +456,50 @@ def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False
         res["through_registry_op"] = bench_registry_op(torch, hidden, weight, targets, grad, temp, ign,
                                                        max(3, steps // 2))
     return res
+
+
+def bench_skip_masked(torch, hidden, weight, targets, mask, old, ref, rewards, grpo, temp, steps):
+    """The GRPO step through the caller-side glue (`training.grpo_loss_step`, autograd), once with
+    every position carried through the kernels and once with the masked positions taken out
+    (`skip_masked`): the same values to fp32 rounding; the work shrinks by the masked share."""
+    from rl_kernel_amd.training import grpo_loss_step
+
+    g, t = grpo["group"], grpo["seq"]
+    head = torch.nn.Linear(1, 1, bias=False)
+    head.in_features, head.out_features = weight.shape[1], weight.shape[0]
+    head.weight = torch.nn.Parameter(weight)  # shares the storage
+    hid = hidden.view(g, t, -1).detach().requires_grad_(True)
+    ids = torch.where(mask, targets.view(g, t), torch.zeros_like(targets.view(g, t)))
+    out = {"active_tokens": int(mask.sum().item()), "tokens": int(mask.numel())}
+    keep = {}
+    for key, skip in (("all_positions_ms", False), ("skip_masked_ms", True)):
+        def step():
+            hid.grad = None
+            head.weight.grad = None
+            r = grpo_loss_step(hid, head, ids, mask, old, ref, rewards, samples_per_prompt=g,
+                               clip_eps=grpo["clip_eps"], beta=grpo["beta"], temperature=temp,
+                               skip_masked=skip)
+            r.loss.backward()
+            return r
+        step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            r = step()
+        torch.cuda.synchronize()
+        out[key] = (time.perf_counter() - t0) * 1e3 / steps
+        keep[key] = (r.loss.detach().clone(), r.current_logps.detach().clone(), hid.grad.clone())
+    a, b = keep["all_positions_ms"], keep["skip_masked_ms"]
+    rel = lambda x, y: float((x.float() - y.float()).norm() / y.float().norm())
+    out["difference"] = {"loss_abs": abs(float(a[0]) - float(b[0])),
+                         "logp_max_abs": float((a[1] - b[1]).abs().max()),
+                         "dH_rel_norm": rel(b[2], a[2])}
+    out["note"] = ("wall clock per step through autograd, bf16 dW returned (the fp32 dW is cast); "
+                   "skip_masked gathers the unmasked rows, runs the head's kernels on them and puts "
+                   "the results back; tokens/s of the headline counts every position as computed "
+                   "and is NOT taken from this mode")
+    head.weight.grad = None
+    return out
 
 
 def bench_registry_op(torch, hidden, weight, targets, grad, temp, ign, steps):

@@ -7,6 +7,7 @@
 // forward and in the dZ recompute M = vocab and N = token, so one lane owns whole token columns
 // and the softmax reduction over vocab is a plain in-register loop with no cross-lane traffic.
 #include "rlk_common.hpp"
+#include <algorithm>
 #include <mutex>
 #include <vector>
 
@@ -952,19 +953,43 @@ int patch_rows_for(int H)
     return H <= 4096 ? 8 : (H <= 8192 ? 4 : 2);
 }
 
+// Vocab splits of one forward launch.  The launch is row_blocks x splits workgroups, one per CU at
+// a time, each walking ceil(tiles / splits) vocab tiles: it takes ceil(workgroups / 256) rounds of
+// the 256 CUs, so a count that lands just above a multiple of 256 wastes most of a round (88 token
+// blocks x 6 splits = 528 workgroups ran three rounds for the work of two).  Among the counts that
+// leave every workgroup a run of at least 8 tiles, those within 2 % of the lowest
+// rounds x (run + half a tile of start-up and state flush) are equally good, and of them the one
+// closest to 512 workgroups (two rounds: the second evens out what the first left uneven) wins.
 int split_count(int row_blocks, int tiles, int patch_rows)
 {
     if (tiles <= 0) return 0;
-    int s = (512 + row_blocks / 2) / row_blocks;
     // At least 32 / patch_rows splits when each still gets a long run of tiles: the 32 workgroups
     // resident on one XCD then form a compact (token blocks x splits) patch that fetches 12 distinct
     // operand streams into its L2 (8 x 4 or 4 x 8) instead of 18 (16 x 2) or 33 (32 x 1).
     const int want = 32 / patch_rows;
-    if (s < want && tiles >= want * 16) s = want;
-    if (s < 1) s = 1;
-    if (s > 64) s = 64;
-    if (s > tiles) s = tiles;
-    return s;
+    const int lo = tiles >= want * 16 ? want : 1;
+    const int hi = tiles < 64 ? tiles : 64;
+    auto cost = [&](int s) {
+        const int64_t run = (tiles + s - 1) / s;
+        const int64_t rounds = (static_cast<int64_t>(row_blocks) * s + 255) / 256;
+        return rounds * (2 * run + 1);
+    };
+    auto allowed = [&](int s) { return s == lo || (tiles + s - 1) / s >= 8; };
+    int64_t lowest = cost(lo);
+    for (int s = lo + 1; s <= hi; ++s)
+        if (allowed(s)) lowest = std::min(lowest, cost(s));
+    int best = lo;
+    int64_t best_dist = -1;
+    for (int s = lo; s <= hi; ++s) {
+        if (!allowed(s) || cost(s) * 100 > lowest * 102) continue;
+        const int64_t wgs = static_cast<int64_t>(row_blocks) * s;
+        const int64_t dist = wgs > 512 ? wgs - 512 : 512 - wgs;
+        if (best_dist < 0 || dist < best_dist) {
+            best = s;
+            best_dist = dist;
+        }
+    }
+    return best;
 }
 
 FwdPlan fwd_plan(int64_t N, int H, int64_t V, bool all_general)

@@ -54,6 +54,25 @@ def _check_grad_buffer(name: str, buf: torch.Tensor, shape, device) -> None:
         raise ValueError(f"{name} must not require grad (it is a gradient buffer)")
 
 
+def _compact_rows(hidden: torch.Tensor, target_ids: torch.Tensor, ignore_index: int):
+    """``(rows, hidden[rows], targets[rows])`` for the rows whose target is not ``ignore_index``,
+    or ``None`` when no row or every row would be kept (then there is nothing to gain, and an
+    empty block would cut the result off the autograd graph).  ``rows`` (flat indices) is filled up
+    to a multiple of 256 with ignored rows, which cost a fraction of a tile and keep the block on
+    the kernels' full-tile routes; they come back as the zeros they are."""
+    flat = target_ids.reshape(-1).to(device=hidden.device)
+    keep = flat != ignore_index
+    rows = torch.nonzero(keep).squeeze(1)  # synchronises: the count sizes the launches
+    n_keep = rows.numel()
+    if n_keep == 0 or n_keep == flat.numel():
+        return None
+    fill = min(-n_keep % 256, flat.numel() - n_keep)
+    if fill:
+        rows = torch.cat([rows, torch.nonzero(~keep).squeeze(1)[:fill]])
+    hidden_2d = hidden.reshape(-1, hidden.size(-1))
+    return rows, hidden_2d.index_select(0, rows), flat.index_select(0, rows)
+
+
 def hip_path_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     """bf16 / f16 / f32 tensors of one dtype on one GPU.  bf16/f16 with a hidden size that is a
     multiple of 8 run on the 16-bit MFMA tiles, the rest on the fp32 matrix-core kernels."""
@@ -530,21 +549,34 @@ class RocmFusedLinearLogpOp:
                  check_targets: bool = True, norm_weight: Optional[torch.Tensor] = None,
                  norm_eps: float = 1e-6, weight_grad_out: Optional[torch.Tensor] = None,
                  bias_grad_out: Optional[torch.Tensor] = None,
-                 accumulate: bool = True) -> torch.Tensor:
+                 accumulate: bool = True, compact_ignored: bool = False) -> torch.Tensor:
         return self.apply(hidden, lm_head_weight, target_ids, bias, tp_group=tp_group,
                           vocab_start_index=vocab_start_index, global_vocab_size=global_vocab_size,
                           temperature=temperature, ignore_index=ignore_index,
                           check_targets=check_targets, norm_weight=norm_weight, norm_eps=norm_eps,
                           weight_grad_out=weight_grad_out, bias_grad_out=bias_grad_out,
-                          accumulate=accumulate)
+                          accumulate=accumulate, compact_ignored=compact_ignored)
 
     def apply(self, hidden, lm_head_weight, target_ids, bias=None, *, tp_group: Any = None,
               vocab_start_index: int = 0, global_vocab_size: Optional[int] = None,
               temperature: float = 1.0, ignore_index: Optional[int] = None,
               check_targets: bool = True, norm_weight: Optional[torch.Tensor] = None,
               norm_eps: float = 1e-6, weight_grad_out: Optional[torch.Tensor] = None,
-              bias_grad_out: Optional[torch.Tensor] = None, accumulate: bool = True) -> torch.Tensor:
+              bias_grad_out: Optional[torch.Tensor] = None, accumulate: bool = True,
+              compact_ignored: bool = False) -> torch.Tensor:
         """Selected-token log-prob in float32 with the leading shape of ``hidden``.
+
+        ``compact_ignored`` (keyword-only, default off; needs ``ignore_index``): the rows whose
+        target is ``ignore_index`` (prompt and padding positions of an RL batch) are left out of
+        the kernels instead of being carried through them as rows of zeros: the other rows are
+        gathered into a dense ``[n_active, H]`` block, the forward and the backward run on that
+        block, and the results are put back (ignored positions: log-prob 0, zero hidden gradient,
+        no contribution to the weight gradient, as without the option).  Rows do not interact, so
+        the results are the same numbers; they are not always the same bits, because the number of
+        vocab splits, token chunks and vocab pieces follows the row count and the fp32 sums are
+        then grouped differently (log-probs agree to about 1e-6, gradients to one rounding of
+        their output type).  Costs one host synchronisation (the launch sizes depend on the
+        count) and the gathered block, ``n_active * H`` elements held until the backward.
 
         ``weight_grad_out`` / ``bias_grad_out`` (keyword-only, default off): contiguous float32
         ``[V, H]`` / ``[V]`` buffers of the caller (fp32 main gradients).  The backward then adds
@@ -606,6 +638,17 @@ class RocmFusedLinearLogpOp:
                 _check_grad_buffer(name, buf, shape, hidden.device)
         if bias_grad_out is not None and bias is None:
             raise ValueError("bias_grad_out given without a bias")
+        if compact_ignored and ignore_index is not None:
+            compact = _compact_rows(hidden, target_ids, ignore_index)
+            if compact is not None:
+                rows, hidden_c, target_c = compact
+                logp_c = self.apply(hidden_c, lm_head_weight, target_c, bias, temperature=temperature,
+                                    ignore_index=ignore_index, check_targets=check_targets,
+                                    norm_weight=norm_weight, norm_eps=norm_eps,
+                                    weight_grad_out=weight_grad_out, bias_grad_out=bias_grad_out,
+                                    accumulate=accumulate)
+                full = logp_c.new_zeros(target_ids.numel()).index_copy(0, rows, logp_c)
+                return full.reshape(target_ids.shape)
         if norm_weight is not None:
             if weight_grad_out is not None or bias_grad_out is not None:
                 raise NotImplementedError("weight_grad_out / bias_grad_out are not wired into the "

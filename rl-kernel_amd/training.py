@@ -161,16 +161,18 @@ def safe_token_ids(token_ids: torch.Tensor, mask: Optional[torch.Tensor] = None)
 
 def extract_logps(hidden: Any, lm_head: torch.nn.Module, token_ids: torch.Tensor,
                   completion_mask: Optional[torch.Tensor], linear_logp_op: Any, *,
-                  temperature: float = 1.0, output_dtype: torch.dtype = torch.float32
-                  ) -> torch.Tensor:
+                  temperature: float = 1.0, output_dtype: torch.dtype = torch.float32,
+                  skip_masked: bool = True) -> torch.Tensor:
     """Selected-token log-probs of ``lm_head(hidden)`` with masked positions exactly 0.
 
     ``hidden`` is the hidden-state tensor or any model output ``extract_hidden_states`` accepts;
     ``lm_head`` is the head (``torch.nn.Linear``) or, as in the reference's ``_extract_logps``, the
     model that exposes it as ``.lm_head``.  With an op that understands ``ignore_index`` (the HIP
-    backend) masked positions are marked ``-100`` and skipped inside the kernel; with any other
-    ``linear_logp`` backend the reference's two-pass convention is used (safe ids, then
-    ``masked_fill``)."""
+    backend) masked positions are marked ``-100``; with ``skip_masked`` the op then runs its
+    kernels on the unmasked rows only (``compact_ignored``: the same values to fp32 rounding,
+    the masked share of the work saved), without it they pass through the kernels as rows that
+    produce 0 and no gradient.  With any other ``linear_logp`` backend the reference's two-pass
+    convention is used (safe ids, then ``masked_fill``)."""
     if not isinstance(lm_head, torch.nn.Linear):
         lm_head = getattr(lm_head, "lm_head", None)
     if not isinstance(lm_head, torch.nn.Linear):
@@ -186,7 +188,8 @@ def extract_logps(hidden: Any, lm_head: torch.nn.Module, token_ids: torch.Tensor
             active = completion_mask.to(device=ids.device, dtype=torch.bool)
             marked = marked.masked_fill(~active, IGNORE_INDEX)
         logps = linear_logp_op(hidden, lm_head.weight, marked, lm_head.bias,
-                               temperature=temperature, ignore_index=IGNORE_INDEX)
+                               temperature=temperature, ignore_index=IGNORE_INDEX,
+                               compact_ignored=skip_masked and completion_mask is not None)
     else:
         if temperature != 1.0:
             raise ValueError("only the fused HIP backend takes a temperature")
@@ -211,11 +214,15 @@ def grpo_loss_step(hidden: torch.Tensor, lm_head: torch.nn.Linear, token_ids: to
                    ref_logps: Optional[torch.Tensor], rewards: torch.Tensor, *,
                    samples_per_prompt: Optional[int] = None, group_boundaries=None,
                    clip_eps: float = 0.2, beta: float = 0.0, temperature: float = 1.0,
-                   registry=None, fuse_epilogue: bool = True) -> GRPOStepResult:
+                   registry=None, fuse_epilogue: bool = True,
+                   skip_masked: bool = False) -> GRPOStepResult:
     """hidden -> fused logp -> group-normalised advantages -> fused GRPO loss (call
     ``result.loss.backward()`` for dH / dW / db).  Ops come from the kernel registry.  With
     ``fuse_epilogue`` (hidden states and head of one dtype on the GPU) the loss terms leave the
-    forward's last launch (``grpo_step_from_hidden``); the values are the same bits either way."""
+    forward's last launch (``grpo_step_from_hidden``); the values are the same bits either way.
+    ``skip_masked`` takes the positions outside ``completion_mask`` out of the head's kernels
+    (see ``extract_logps``; the loss then comes from the stand-alone epilogue): the step gets
+    cheaper by about the masked share of the batch, and the values agree to fp32 rounding."""
     if registry is None:
         from .registry import kernel_registry as registry
     linear_logp = registry.get_op("linear_logp")
@@ -225,7 +232,8 @@ def grpo_loss_step(hidden: torch.Tensor, lm_head: torch.nn.Linear, token_ids: to
     if not isinstance(lm_head, torch.nn.Linear):
         raise TypeError("model must expose an lm_head torch.nn.Linear for linear_logp")
     hidden = extract_hidden_states(hidden, expected_hidden_dim=int(lm_head.in_features))
-    fusable = (fuse_epilogue and hidden.dim() >= 2 and lm_head.weight.dtype == hidden.dtype
+    fusable = (fuse_epilogue and not (skip_masked and completion_mask is not None)
+               and hidden.dim() >= 2 and lm_head.weight.dtype == hidden.dtype
                and hidden.dtype in (torch.bfloat16, torch.float16, torch.float32))
     if fusable:
         step_op = registry.get_op("grpo_step_from_hidden")
@@ -236,7 +244,7 @@ def grpo_loss_step(hidden: torch.Tensor, lm_head: torch.nn.Linear, token_ids: to
                                      temperature=temperature)
         return GRPOStepResult(loss, pol, kl, cur, adv)
     cur = extract_logps(hidden, lm_head, token_ids, completion_mask, linear_logp,
-                        temperature=temperature)
+                        temperature=temperature, skip_masked=skip_masked)
     adv = loss_op.group_advantages(rewards, samples_per_prompt=samples_per_prompt,
                                    group_boundaries=group_boundaries)
     loss, pol, kl = loss_op(cur, old_logps, ref_logps, adv, completion_mask, clip_eps=clip_eps,

@@ -89,6 +89,25 @@ def test_forward_workspace_is_small(native):
     assert 0 < need.value <= 64 << 20
 
 
+def test_forward_split_count_fills_whole_rounds_of_the_chip(native):
+    """The forward launches (token blocks x vocab splits) workgroups, one per CU at a time.  For any
+    token count the split count must not leave most of a round of the 256 CUs idle: modelled
+    occupancy (work / rounds x longest run) stays above 90 % from 8 token blocks on.  Read back
+    through the workspace size (3 floats per token and split) at the Llama head, whose 501 vocab
+    tiles are all full."""
+    lib = native.load()
+    tiles = 128256 // 256
+    for blocks in range(8, 513):
+        n = blocks * 256
+        need = ctypes.c_size_t(0)
+        assert lib.rlk_linear_logp_fwd_workspace_bytes(n, 4096, 128256, 0, ctypes.byref(need)) == 0
+        splits = need.value // (12 * n)
+        assert 1 <= splits <= 64 and need.value == 12 * n * splits
+        run = -(-tiles // splits)
+        rounds = -(-(blocks * splits) // 256)
+        assert blocks * tiles / 256 / (rounds * run) > 0.90, (blocks, splits)
+
+
 def test_bad_arguments_are_reported_not_launched(native):
     lib = native.load()
     need = ctypes.c_size_t(0)
