@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "89e08cbb44fc092a",
-    "measured_at_commit": "04fb7f0",
+    "kernel_source_sha16": "0e1edf57a3d12c8d",
+    "measured_at_commit": "13c1314",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 56960450635,
-        "linear_logp_dz_kernel": 1953398134,
-        "linear_logp_dh_kernel": 1836843252,
-        "linear_logp_dw_kernel": 2110189437,
+        "linear_logp_fwd_kernel": 58107689907,
+        "linear_logp_dz_kernel": 1958923406,
+        "linear_logp_dh_kernel": 1835560235,
+        "linear_logp_dw_kernel": 2113569513,
     },
 }
 

@@ -956,37 +956,35 @@ int patch_rows_for(int H)
 // Vocab splits of one forward launch.  The launch is row_blocks x splits workgroups, one per CU at
 // a time, each walking ceil(tiles / splits) vocab tiles: it takes ceil(workgroups / 256) rounds of
 // the 256 CUs, so a count that lands just above a multiple of 256 wastes most of a round (88 token
-// blocks x 6 splits = 528 workgroups ran three rounds for the work of two).  Among the counts that
-// leave every workgroup a run of at least 8 tiles, those within 2 % of the lowest
-// rounds x (run + half a tile of start-up and state flush) are equally good, and of them the one
-// closest to 512 workgroups (two rounds: the second evens out what the first left uneven) wins.
+// blocks x 6 splits = 528 workgroups ran three rounds for the work of two: 976 instead of 1370
+// TFLOP/s).  The count with the lowest rounds x (run + half a tile of start-up and state flush)
+// wins, a smaller one when it is within 1.5 %, among the counts that leave every workgroup a run of
+// at least 8 tiles and keep the split partials (12 bytes per token and split) within the 8 MiB the
+// allocation-free entry point has; measured over 4 - 32 splits at 48 - 243 token blocks, this
+// choice is within 1.5 % of the best count tried.
 int split_count(int row_blocks, int tiles, int patch_rows)
 {
     if (tiles <= 0) return 0;
     // At least 32 / patch_rows splits when each still gets a long run of tiles: the 32 workgroups
     // resident on one XCD then form a compact (token blocks x splits) patch that fetches 12 distinct
-    // operand streams into its L2 (8 x 4 or 4 x 8) instead of 18 (16 x 2) or 33 (32 x 1).
+    // operand streams into its L2 (8 x 4 or 4 x 8) instead of 18 (16 x 2) or 33 (32 x 1); with 243
+    // token blocks, 2 or 3 splits ran at 1160 - 1190 TFLOP/s where 4 ran at 1383.
     const int want = 32 / patch_rows;
     const int lo = tiles >= want * 16 ? want : 1;
-    const int hi = tiles < 64 ? tiles : 64;
-    auto cost = [&](int s) {
-        const int64_t run = (tiles + s - 1) / s;
-        const int64_t rounds = (static_cast<int64_t>(row_blocks) * s + 255) / 256;
-        return rounds * (2 * run + 1);
-    };
-    auto allowed = [&](int s) { return s == lo || (tiles + s - 1) / s >= 8; };
-    int64_t lowest = cost(lo);
-    for (int s = lo + 1; s <= hi; ++s)
-        if (allowed(s)) lowest = std::min(lowest, cost(s));
+    int hi = tiles < 64 ? tiles : 64;
+    const int64_t fit = static_cast<int64_t>(RLK_STATIC_SCRATCH_BYTES) / (3072LL * row_blocks);
+    if (hi > fit) hi = fit > lo ? static_cast<int>(fit) : lo;
     int best = lo;
-    int64_t best_dist = -1;
+    int64_t best_cost = -1;
     for (int s = lo; s <= hi; ++s) {
-        if (!allowed(s) || cost(s) * 100 > lowest * 102) continue;
-        const int64_t wgs = static_cast<int64_t>(row_blocks) * s;
-        const int64_t dist = wgs > 512 ? wgs - 512 : 512 - wgs;
-        if (best_dist < 0 || dist < best_dist) {
+        const int64_t run = (tiles + s - 1) / s;
+        if (s > lo && run < 8) break;
+        const int64_t rounds = (static_cast<int64_t>(row_blocks) * s + 255) / 256;
+        const int64_t cost = rounds * (2 * run + 1);
+        // a larger count has to be 1.5 % better than the best smaller one to replace it
+        if (best_cost < 0 || cost * 1000 < best_cost * 985) {
             best = s;
-            best_dist = dist;
+            best_cost = cost;
         }
     }
     return best;

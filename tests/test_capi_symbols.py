@@ -92,9 +92,10 @@ def test_forward_workspace_is_small(native):
 def test_forward_split_count_fills_whole_rounds_of_the_chip(native):
     """The forward launches (token blocks x vocab splits) workgroups, one per CU at a time.  For any
     token count the split count must not leave most of a round of the 256 CUs idle: modelled
-    occupancy (work / rounds x longest run) stays above 90 % from 8 token blocks on.  Read back
-    through the workspace size (3 floats per token and split) at the Llama head, whose 501 vocab
-    tiles are all full."""
+    occupancy (work / rounds x longest run) stays above 88 % from 8 token blocks on (the former
+    rule fell to 68 % at 88 and 105 blocks), and the split partials stay within the 8 MiB of the
+    allocation-free entry point up to 131072 tokens.  Read back through the workspace size
+    (3 floats per token and split) at the Llama head, whose 501 vocab tiles are all full."""
     lib = native.load()
     tiles = 128256 // 256
     for blocks in range(8, 513):
@@ -105,7 +106,8 @@ def test_forward_split_count_fills_whole_rounds_of_the_chip(native):
         assert 1 <= splits <= 64 and need.value == 12 * n * splits
         run = -(-tiles // splits)
         rounds = -(-(blocks * splits) // 256)
-        assert blocks * tiles / 256 / (rounds * run) > 0.90, (blocks, splits)
+        assert blocks * tiles / 256 / (rounds * run) > 0.88, (blocks, splits)
+        assert need.value <= 8 << 20
 
 
 def test_bad_arguments_are_reported_not_launched(native):
