@@ -338,8 +338,6 @@ def fused_linear_logp_backward(
     v = weight.size(0)
     dev = hidden_2d.device
     dt = _DTYPES[hidden_2d.dtype]
-    g = grad_logp.reshape(-1).to(torch.float32).contiguous()
-    d_hidden = torch.empty_like(hidden_2d) if need_hidden else None
     want_bias = bias is not None and need_bias
     if weight_grad_out is not None:
         _check_grad_buffer("weight_grad_out", weight_grad_out, (v, h), dev)
@@ -356,6 +354,8 @@ def fused_linear_logp_backward(
             int(vocab_start), bool(need_hidden), bool(need_weight), bool(want_bias),
             int(dz_budget_bytes), weight_grad_out, bias_grad_out, bool(accumulate))
         return d_hidden, d_weight, d_bias
+    g = grad_logp.reshape(-1).to(torch.float32).contiguous()
+    d_hidden = torch.empty_like(hidden_2d) if need_hidden else None
     d_weight = None
     if need_weight:
         d_weight = weight_grad_out if weight_grad_out is not None else \

@@ -143,3 +143,32 @@ def test_buffer_argument_errors(dev, op):
         op(hd, wd, td, bias_grad_out=torch.zeros(512, device=dev))
     with pytest.raises(ValueError, match="bias_grad_out"):
         op(hd, wd, td, bd, bias_grad_out=torch.zeros(511, device=dev))
+
+
+def test_backward_holds_nothing_beyond_outputs_and_workspace(dev, op):
+    """Extra device memory while the op's backward runs in main-gradient mode = the library's
+    workspace (rlk_linear_logp_bwd_workspace_bytes), the fp32 copy of the upstream gradient and
+    allocator rounding: no second hidden-sized or weight-sized block."""
+    from rl_kernel_amd import _native
+
+    n, h, v = 8192, 1024, 16384
+    g = torch.Generator().manual_seed(3)
+    hidden = torch.randn(n, h, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
+    weight = (0.05 * torch.randn(v, h, generator=g)).to(torch.bfloat16).to(dev).requires_grad_(True)
+    ids = torch.randint(0, v, (n,), generator=g).to(dev)
+    up = torch.randn(n, generator=g).to(dev)
+    main = torch.zeros(v, h, device=dev)
+    need = ctypes.c_size_t(0)
+    assert _native.load().rlk_linear_logp_bwd_workspace_bytes(n, h, v, 0, 0, ctypes.byref(need)) == 0
+    for _ in range(2):  # the second pass measures: every lazy one-time allocation is behind it
+        hidden.grad = None
+        logp = op(hidden, weight, ids, weight_grad_out=main, check_targets=False)
+        loss = (logp * up).sum()
+        torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated()
+        torch.cuda.reset_peak_memory_stats()
+        loss.backward()
+        torch.cuda.synchronize()
+        extra = torch.cuda.max_memory_allocated() - base
+    d_hidden_bytes = n * h * 2
+    assert extra <= need.value + d_hidden_bytes + (4 << 20), (extra, need.value)
