@@ -2,10 +2,11 @@
 // tiles, logits never stored), split combine, and the recompute-based backward (dZ block,
 // dH and dW contractions).  All reductions run in a fixed order: same input, same bits.
 //
-// Orientation used by every kernel here: the MFMA "M" index lives in accumulator registers
-// (4 consecutive rows per register quad), the "N" index is the lane (column l % 32).  In the
-// forward and in the dZ recompute M = vocab and N = token, so one lane owns whole token columns
-// and the softmax reduction over vocab is a plain in-register loop with no cross-lane traffic.
+// Orientation used by every kernel here: the MFMA "M" index lives in accumulator registers (the
+// 4 registers of a 16 x 16 tile hold rows 4 (l / 16) + 0..3 of column l % 16), the "N" index is
+// the lane.  In the forward and in the dZ recompute M = vocab and N = token, so the softmax
+// reduction over vocab is an in-register loop per lane; the four lanes that share a token column
+// (l, l + 16, l + 32, l + 48) merge their states by two shuffles once per split.
 #include "rlk_common.hpp"
 #include <algorithm>
 #include <mutex>
