@@ -43,14 +43,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "f6136cca09e1e933",
-    "measured_at_commit": "36a2ee8",
+    "kernel_source_sha16": "a7c983286935f1d1",
+    "measured_at_commit": "93d5cb2",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 53562865536,
-        "linear_logp_dz_kernel": 1957185679,
-        "linear_logp_dh_kernel": 1832259844,
-        "linear_logp_dw_kernel": 2108853750,
+        "linear_logp_fwd_kernel": 63292998433,
+        "linear_logp_dz_kernel": 1956222218,
+        "linear_logp_dh_kernel": 1835825439,
+        "linear_logp_dw_kernel": 2109236135,
     },
 }
 
