@@ -23,7 +23,6 @@ Prints ONE JSON line.  Besides the headline metric (tokens/s of the whole step) 
 from __future__ import annotations
 
 import argparse
-import glob
 import hashlib
 import json
 import os
@@ -89,14 +88,18 @@ REFERENCE_PUBLISHED_H100 = {
 }
 
 
+KERNEL_SOURCES = ("rlk_common.hpp", "rlk_gemm.hpp", "rlk_grpo.hpp", "rlk_linear_logp.hip",
+                  "rlk_tile_epilogue.hpp")
+
+
 def kernel_source_sha16() -> str:
-    """Digest of the device-code sources (kernels and their headers; the PyTorch binding is host
-    code only)."""
+    """Digest of the sources the four contraction kernels are compiled from (the file that holds
+    them and the headers it includes)."""
     m = hashlib.sha256()
     csrc = os.path.join(ROOT, "rl-kernel_amd", "csrc")
-    for path in sorted(glob.glob(os.path.join(csrc, "*.hip")) + glob.glob(os.path.join(csrc, "*.hpp"))):
-        with open(path, "rb") as fh:
-            m.update(os.path.basename(path).encode())
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(csrc, name), "rb") as fh:
+            m.update(name.encode())
             m.update(fh.read())
     return m.hexdigest()[:16]
 
@@ -159,12 +162,20 @@ def cpu_baseline(torch, cfg, slice_tokens, iters=2):
 
 
 def device_info(torch):
+    """Name, compute units and maximum engine clock as the HIP runtime reports them, and the 16-bit
+    matrix-core peak they imply (CU x 4096 flop per clock x clock) next to the published one."""
+    import ctypes
+
+    from rl_kernel_amd import _native
+
     p = torch.cuda.get_device_properties(0)
-    khz = getattr(p, "clock_rate", 0)  # kHz where this torch build exposes it
     info = {"name": p.name, "compute_units": p.multi_processor_count}
-    if khz:
-        info["max_sclk_mhz"] = khz / 1e3
-        info["peak_from_cu_clock_tflops"] = p.multi_processor_count * 4096 * khz * 1e3 / 1e12
+    cu, khz = ctypes.c_int32(0), ctypes.c_int32(0)
+    if _native.load().rlk_device_info(0, ctypes.byref(cu), ctypes.byref(khz)) == 0 and khz.value > 0:
+        info["compute_units"] = cu.value
+        info["max_sclk_mhz"] = khz.value / 1e3
+        info["peak_from_cu_clock_tflops"] = cu.value * 4096 * khz.value * 1e3 / 1e12
+        info["published_peak_tflops"] = PEAK_TFLOPS["bf16"]
     return info
 
 

@@ -48,6 +48,11 @@ int rlk_version(void);
  * until the next failing call on the same thread. */
 const char* rlk_last_error(void);
 
+/* Compute units and maximum engine clock (kHz) of HIP device `device`, as the runtime reports
+ * them: what a benchmark prices the matrix-core peak with (compute units x 4096 flop per clock x
+ * clock for 16-bit inputs).  No counterpart in the reference.  Host pointers; launches nothing. */
+int rlk_device_info(int32_t device, int32_t* compute_units, int32_t* max_clock_khz);
+
 /* ------------------------------------------------------------------------------------------ *
  * Fused linear -> selected-token log-prob, forward.
  *

@@ -17,6 +17,7 @@ _vp, _i32, _i64, _sz, _f32 = _c.c_void_p, _c.c_int32, _c.c_int64, _c.c_size_t, _
 # name -> (restype, argtypes); mirrors include/rlk_hip.h one to one
 SIGNATURES = {
     "rlk_version": (_c.c_int, []),
+    "rlk_device_info": (_c.c_int, [_i32, _vp, _vp]),
     "rlk_last_error": (_c.c_char_p, []),
     "rlk_linear_logp_fwd_workspace_bytes": (_c.c_int, [_i64, _i32, _i64, _i32, _c.POINTER(_sz)]),
     "rlk_linear_logp_fwd": (_c.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i32, _i64,
