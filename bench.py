@@ -42,14 +42,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "a7c983286935f1d1",
-    "measured_at_commit": "93d5cb2",
+    "kernel_source_sha16": "9336dbfd8cae79be",
+    "measured_at_commit": "a2945f3",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 63292998433,
-        "linear_logp_dz_kernel": 1956222218,
-        "linear_logp_dh_kernel": 1835825439,
-        "linear_logp_dw_kernel": 2109236135,
+        "linear_logp_fwd_kernel": 58078498827,
+        "linear_logp_dz_kernel": 1955615969,
+        "linear_logp_dh_kernel": 1838319598,
+        "linear_logp_dw_kernel": 2111721843,
     },
 }
 
