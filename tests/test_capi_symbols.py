@@ -126,6 +126,7 @@ def test_bad_arguments_are_reported_not_launched(native):
     assert lib.rlk_grpo_loss_from_logp(None, None, None, None, 1, None, 4, 4, 0.2, 0.0, None, None,
                                        None, None, None, None, None, 0, None) == -1
     assert lib.rlk_group_advantages(None, None, 2, 1e-6, None, None) == -1
+    assert lib.rlk_device_info(0, None, None) == -1 and b"rlk_device_info" in lib.rlk_last_error()
     rc = lib.rlk_linear_logp_fwd(None, None, None, None, None, None, None, 0, 16, 64, 32, 0, 0, 0.0,
                                  0, 0, 1, None, None)
     assert rc == -1 and b"temperature" in lib.rlk_last_error()

@@ -165,3 +165,14 @@ def test_registry_dispatches_to_hip_backends(dev):
     assert kernel_registry.get_op("logp") is kernel_registry.get_op("logp_online")
     with pytest.raises(RuntimeError, match="No functional backend"):
         kernel_registry.get_op("attn")
+
+
+def test_device_info_reports_what_the_runtime_knows(dev):
+    import ctypes
+
+    from rl_kernel_amd import _native
+
+    cu, khz = ctypes.c_int32(0), ctypes.c_int32(0)
+    assert _native.load().rlk_device_info(dev.index or 0, ctypes.byref(cu), ctypes.byref(khz)) == 0
+    assert cu.value == torch.cuda.get_device_properties(dev).multi_processor_count
+    assert 500_000 < khz.value < 5_000_000  # kHz
