@@ -43,13 +43,13 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
     "kernel_source_sha16": "9336dbfd8cae79be",
-    "measured_at_commit": "a2945f3",
+    "measured_at_commit": "52c38ec",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 58078498827,
-        "linear_logp_dz_kernel": 1955615969,
-        "linear_logp_dh_kernel": 1838319598,
-        "linear_logp_dw_kernel": 2111721843,
+        "linear_logp_fwd_kernel": 59135013663,
+        "linear_logp_dz_kernel": 1954204941,
+        "linear_logp_dh_kernel": 1835375736,
+        "linear_logp_dw_kernel": 2109452763,
     },
 }
 
