@@ -155,8 +155,9 @@ int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t
 /* Schedule the backward will use for these sizes (no counterpart in the reference, whose chunk is
  * fixed at 2^24 / V tokens, rl_engine/kernels/ops/pytorch/loss/linear_logp.py:398-400):
  * out5 = { tokens per chunk, vocab rows per piece, number of chunks, number of pieces, parts the
- * dH launch cuts a piece's vocab range into (1 unless there are few tokens) }.  Host only;
- * touches no device. */
+ * dH launch of a full block cuts the piece's vocab range into (1 unless there are few tokens; a
+ * shorter last chunk or piece takes its own count by the same rule) }.  Host only; touches no
+ * device. */
 int rlk_linear_logp_bwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype,
                              size_t dz_budget_bytes, int64_t* out5);
 

@@ -1024,7 +1024,8 @@ struct BwdPlan {
     int v_piece;     // vocab rows per piece (multiple of 256)
     int n_chunks;
     int n_pieces;
-    int ksplit;      // dH launch: parts of the piece's vocab range computed side by side
+    int ksplit;      // dH launch of a full block: parts of the piece's vocab range computed side by
+                     // side; a shorter last chunk / last piece takes its own count (dh_parts)
     int64_t ldz;     // elements between consecutive token rows of the dZ block
     size_t dz_bytes;
     size_t acc_bytes;
@@ -1133,7 +1134,16 @@ BwdPlan bwd_plan(int64_t N, int H, int64_t V, size_t budget)
     // Few tokens: the dH launch has fewer tiles than the chip has CUs but a long vocab range, so
     // the range is cut into parts that run side by side and are added up in a fixed order.
     p.ksplit = dh_parts(best_ct, best_pt, ht);
-    p.part_bytes = p.ksplit > 1 ? static_cast<size_t>(p.ksplit) * p.tok_chunk * H * 4 : 0;
+    // fp32 slots of the split dH launches: every (chunk, piece) kind picks its own part count, so
+    // a short last chunk does not run its few tiles on a quarter of the chip
+    const int64_t ct_last = n_t - (p.n_chunks - 1) * best_ct, pt_last = v_t - (p.n_pieces - 1) * best_pt;
+    p.part_bytes = 0;
+    for (int64_t ct : {best_ct, ct_last})
+        for (int64_t pt : {best_pt, pt_last}) {
+            const int parts = dh_parts(ct, pt, ht);
+            if (parts > 1)
+                p.part_bytes = std::max(p.part_bytes, static_cast<size_t>(parts) * ct * 256 * H * 4);
+        }
     p.part_off = p.acc_off + align_up(p.acc_bytes, 256);
     // per-token-tile column sums of the dZ block (d_bias): 1 KiB per dZ tile
     p.db_bytes = static_cast<size_t>(best_ct) * p.v_piece * 4;
@@ -1327,9 +1337,11 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             h.h_tiles = h_tiles;
             h.first = pi == 0;
             h.last = last_piece;
-            h.ksplit = p.ksplit;
-            h.part = p.ksplit > 1 ? reinterpret_cast<float*>(ws + p.part_off) : nullptr;
-            h.part_stride = static_cast<int64_t>(p.tok_chunk) * H;
+            // same rule as the plan's cost model: per (chunk, piece) kind
+            const int ksplit = dh_parts(tok_tiles, v_tiles, h_tiles);
+            h.ksplit = ksplit;
+            h.part = ksplit > 1 ? reinterpret_cast<float*>(ws + p.part_off) : nullptr;
+            h.part_stride = static_cast<int64_t>(tok_tiles) * 256 * H;
 
             DwArgs d;
             d.dz = dz;
@@ -1370,18 +1382,18 @@ int bwd_enqueue(const BwdCall& c, const BwdPlan& p, int n_cu)
             }
             if (dh) {
                 const int tiles = tok_tiles * h_tiles;
-                if (p.ksplit == 1 && H >= 256 && v_valid % kBK == 0 && v_valid >= 2 * kBK) {
+                if (ksplit == 1 && H >= 256 && v_valid % kBK == 0 && v_valid >= 2 * kBK) {
                     hipLaunchKernelGGL((linear_logp_dh_kernel<T, kBK, true>),
                                        dim3(chain_grid(tiles, n_cu)), dim3(kThreads), kChainSmem,
                                        stream, h);
                 } else {
                     hipLaunchKernelGGL((linear_logp_dh_kernel<T, kBK, false>),
-                                       dim3(tiles * p.ksplit), dim3(kThreads), GH::kSmemBytes, stream, h);
-                    if (p.ksplit > 1) {
+                                       dim3(tiles * ksplit), dim3(kThreads), GH::kSmemBytes, stream, h);
+                    if (ksplit > 1) {
                         const int64_t n4 = static_cast<int64_t>(tok_valid) * H / 4;
                         hipLaunchKernelGGL((linear_logp_dh_reduce_kernel<T>),
                                            dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0,
-                                           stream, h.part, p.ksplit, h.part_stride, h.acc, h.out,
+                                           stream, h.part, ksplit, h.part_stride, h.acc, h.out,
                                            scales, n4, h.first, h.last);
                     }
                 }

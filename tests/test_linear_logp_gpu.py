@@ -527,3 +527,33 @@ def test_few_tokens_long_vocab_split_dh(dev, n, h, v, dtype, budget):
     assert rel(dh, r_dh) < GRAD_REL and rel(dw, r_dw) < GRAD_REL
     assert torch.equal(dh, dh2) and torch.equal(dw, dw2)
     assert torch.all(dh.float().cpu()[tgt == -100] == 0)
+
+
+@pytest.mark.parametrize("n,h,v,budget,chunks,pieces", [
+    # 16 + 5 token tiles x 32 + 16 vocab tiles: the long pieces run the split dH launch (2 parts),
+    # the short last piece the chained walk, and both feed one fp32 accumulator per chunk
+    (5376, 2048, 12288, 64 << 20, 2, 2),
+    # 17 + 16 token tiles over one 64-tile piece: 2 parts for the first chunk, 4 for the last
+    (8448, 1024, 16384, 0, 2, 1),
+])
+def test_dh_part_count_follows_each_chunk_and_piece(dev, n, h, v, budget, chunks, pieces):
+    """The dH launch of every (token chunk, vocab piece) block picks its own number of side-by-side
+    parts, so a short last chunk or piece is not run with the count of the full block."""
+    import ctypes
+
+    from rl_kernel_amd import _native
+    from rl_kernel_amd.ops import linear_logp as LL
+
+    plan = (ctypes.c_int64 * 5)()
+    assert _native.load().rlk_linear_logp_bwd_plan(n, h, v, 0, budget, plan) == 0
+    assert (plan[2], plan[3]) == (chunks, pieces), list(plan)
+    hidden, weight, _, tgt, grad = make(47, (n,), h, v, torch.bfloat16, False, 0.05)
+    r_dh, r_dw, _ = O.linear_logp_backward(grad, hidden, weight, tgt, ignore_index=-100, token_chunk=2048)
+    hd, wd, td = hidden.to(dev), weight.to(dev), tgt.to(dev)
+    _, lse, _ = LL.fused_linear_logp_forward(hd, wd, td, ignore_index=-100)
+    outs = [LL.fused_linear_logp_backward(grad.to(dev), hd, wd, td, lse, ignore_index=-100,
+                                          dz_budget_bytes=budget) for _ in range(2)]
+    dh, dw = outs[0][0], outs[0][1]
+    assert rel(dh, r_dh) < GRAD_REL and rel(dw, r_dw) < GRAD_REL
+    assert torch.equal(dh, outs[1][0]) and torch.equal(dw, outs[1][1])
+    assert torch.all(dh.float().cpu()[tgt == -100] == 0)
