@@ -82,6 +82,51 @@ def test_backward_plan_covers_the_problem_within_budget(native, n, h, v, budget)
     assert _plan(lib, n, h, v, 0, budget) == (tok_chunk, v_piece, n_chunks, n_pieces, dh_parts)  # memoised
 
 
+def _dh_parts(ct, pt, ht):
+    """The library's rule for the side-by-side parts of a dH launch (restated from its text in
+    include/rlk_hip.h and the kernel file: at most 128 tiles, a vocab range of at least 32 tiles,
+    a power of two up to 8 that keeps the launch within 256 workgroups and 16 tiles per part)."""
+    tiles, parts = ct * ht, 1
+    if tiles <= 128 and pt >= 32:
+        lim = min(256 // tiles, pt // 16, 8)
+        while parts * 2 <= lim:
+            parts *= 2
+    return parts
+
+
+def test_backward_workspace_holds_the_dh_slots_of_every_block_kind(native):
+    """A shorter last chunk or piece picks its own dH part count; the workspace must hold the fp32
+    slots of whichever (chunk, piece) kind needs most, next to the dZ block, the fp32 dH
+    accumulator and the d_bias column sums."""
+    import random
+
+    lib = native.load()
+    rng = random.Random(7)
+    for _ in range(400):
+        n = rng.randrange(1, 140) * 256 - rng.randrange(0, 256)
+        h = rng.choice((64, 256, 896, 1024, 2048, 4096, 8192))
+        v = rng.randrange(300, 160000)
+        budget = rng.choice((0, 16 << 20, 64 << 20, 128 << 20))
+        tok_chunk, v_piece, n_chunks, n_pieces, parts_full = _plan(lib, n, h, v, 0, budget)
+        ct, pt, ht = tok_chunk // 256, v_piece // 256, (h + 255) // 256
+        n_t, v_t = (n + 255) // 256, (v + 255) // 256
+        ct_last, pt_last = n_t - (n_chunks - 1) * ct, v_t - (n_pieces - 1) * pt
+        assert parts_full == _dh_parts(ct, pt, ht)
+        slots = 0
+        for c in (ct, ct_last):
+            for p_ in (pt, pt_last):
+                k = _dh_parts(c, p_, ht)
+                if k > 1:
+                    slots = max(slots, k * c * 256 * h * 4)
+        need = ctypes.c_size_t(0)
+        assert lib.rlk_linear_logp_bwd_workspace_bytes(n, h, v, 0, budget, ctypes.byref(need)) == 0
+        dz = tok_chunk * v_piece * 2
+        acc = tok_chunk * h * 4 if n_pieces > 1 else 0
+        db = ct * v_piece * 4
+        assert need.value >= 256 + dz + acc + slots + db, (n, h, v, budget)
+        assert slots <= 67 << 20  # <= 256 tiles of fp32
+
+
 def test_forward_workspace_is_small(native):
     lib = native.load()
     need = ctypes.c_size_t(0)
