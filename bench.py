@@ -238,6 +238,18 @@ def bwd_plan(n, h, v, dtype_id):
     return dict(tok_chunk=out[0], v_piece=out[1], n_chunks=out[2], n_pieces=out[3], dh_parts=out[4])
 
 
+def fwd_plan(n, h, v, dtype_id):
+    import ctypes
+
+    from rl_kernel_amd import _native
+
+    out = (ctypes.c_int64 * 4)()
+    _native.check(_native.load().rlk_linear_logp_fwd_plan(n, h, v, dtype_id, out), "plan")
+    wgs = out[0] * out[1]
+    return dict(token_blocks=out[0], vocab_splits=out[1], ragged_tile_splits=out[2],
+                token_blocks_per_xcd_patch=out[3], workgroups=wgs, rounds_of_256_cus=wgs / 256.0)
+
+
 def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False, registry_op=False,
                  probe_epilogue=True, kernel_timing=True):
     """Forward(+backward) of the fused LM-head logp through the raw C-ABI wrappers."""
@@ -438,6 +450,7 @@ def bench_linear(torch, name, cfg, steps, warmup, mode="fwd+bwd", detailed=False
                             "achieved": blk_flops / (total / blocks * 1e-3) / 1e12,
                             "algorithmic_bytes": float(alg[kname])})
         res["backward_plan"] = plan
+        res["forward_plan"] = fwd_plan(n, h, v, 0 if cfg["dtype"] == "bf16" else 1)
         res["backward_ms"] = t_all
         res["kernel_timing_method"] = (
             "HIP events on the launch stream; forward alone; backward kernels from three backward "

@@ -41,7 +41,8 @@ enum {
     RLK_ERR_LAUNCH = -3       /* HIP refused the launch */
 };
 
-/* ABI version of this header (major * 100 + minor). */
+/* ABI version of this header (major * 100 + minor): 101 (100 + rlk_device_info and
+ * rlk_linear_logp_fwd_plan). */
 int rlk_version(void);
 
 /* Message of the last error returned on the calling thread ("" if none). Host pointer, valid
@@ -83,6 +84,16 @@ int rlk_device_info(int32_t device, int32_t* compute_units, int32_t* max_clock_k
  * ------------------------------------------------------------------------------------------ */
 int rlk_linear_logp_fwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t dtype,
                                         size_t* bytes);
+
+/* Schedule the forward will use for these sizes (the reference computes its own inside the host
+ * function: 4 workgroups per SM divided by the token blocks, csrc/cuda/fused_linear_logp_sm90.cu:
+ * 350-358,369, and does not expose it): out4 = { blocks of 256
+ * tokens, vocab splits of the launch over the full vocab tiles, vocab splits of the launch over
+ * the ragged last tile (all tiles for RLK_DTYPE_F32; 0 if there is no such launch), token blocks
+ * per XCD patch }.  The contraction launches are blocks x splits workgroups.  Inputs whose rows
+ * do not start on 16-byte boundaries run the RLK_DTYPE_F32 schedule.  Host only; touches no
+ * device. */
+int rlk_linear_logp_fwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype, int64_t* out4);
 
 int rlk_linear_logp_fwd(const void* hidden, const void* weight, const float* bias,
                         const int64_t* targets, float* logp, float* lse, void* workspace,

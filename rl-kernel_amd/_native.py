@@ -31,6 +31,7 @@ SIGNATURES = {
                                             _vp]),
     "rlk_linear_logp_bwd_workspace_bytes": (_c.c_int, [_i64, _i32, _i64, _i32, _sz,
                                                        _c.POINTER(_sz)]),
+    "rlk_linear_logp_fwd_plan": (_c.c_int, [_i64, _i32, _i64, _i32, _c.POINTER(_i64)]),
     "rlk_linear_logp_bwd_plan": (_c.c_int, [_i64, _i32, _i64, _i32, _sz, _c.POINTER(_i64)]),
     "rlk_linear_logp_bwd": (_c.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz,
                                        _i64, _i32, _i64, _i64, _i32, _f32, _i64, _i32, _vp]),

@@ -16,7 +16,7 @@ int rlk_fail(int code, const char* msg)
 
 extern "C" {
 
-int rlk_version(void) { return 100; }
+int rlk_version(void) { return 101; }
 
 const char* rlk_last_error(void) { return g_last_error; }
 

@@ -1759,6 +1759,17 @@ int rlk_linear_logp_bwd_workspace_bytes(int64_t N, int32_t H, int64_t V, int32_t
     return 0;
 }
 
+int rlk_linear_logp_fwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype, int64_t* out4)
+{
+    if (!out4 || N <= 0 || V <= 0 || H <= 0) return rlk_fail(RLK_ERR_ARG, "bad plan query");
+    const FwdPlan p = fwd_plan(N, H, V, dtype == RLK_DTYPE_F32);
+    out4[0] = p.row_blocks;
+    out4[1] = p.n_fast;
+    out4[2] = p.n_gen;
+    out4[3] = p.patch_rows;
+    return 0;
+}
+
 int rlk_linear_logp_bwd_plan(int64_t N, int32_t H, int64_t V, int32_t dtype, size_t dz_budget_bytes,
                              int64_t* out5)
 {

@@ -149,6 +149,9 @@ def test_forward_split_count_fills_whole_rounds_of_the_chip(native):
         assert lib.rlk_linear_logp_fwd_workspace_bytes(n, 4096, 128256, 0, ctypes.byref(need)) == 0
         splits = need.value // (12 * n)
         assert 1 <= splits <= 64 and need.value == 12 * n * splits
+        plan = (ctypes.c_int64 * 4)()
+        assert lib.rlk_linear_logp_fwd_plan(n, 4096, 128256, 0, plan) == 0
+        assert tuple(plan) == (blocks, splits, 0, 8)
         run = -(-tiles // splits)
         rounds = -(-(blocks * splits) // 256)
         assert blocks * tiles / 256 / (rounds * run) > 0.88, (blocks, splits)
@@ -172,6 +175,7 @@ def test_bad_arguments_are_reported_not_launched(native):
                                        None, None, None, None, None, 0, None) == -1
     assert lib.rlk_group_advantages(None, None, 2, 1e-6, None, None) == -1
     assert lib.rlk_device_info(0, None, None) == -1 and b"rlk_device_info" in lib.rlk_last_error()
+    assert lib.rlk_linear_logp_fwd_plan(16, 64, 32, 0, None) == -1
     rc = lib.rlk_linear_logp_fwd(None, None, None, None, None, None, None, 0, 16, 64, 32, 0, 0, 0.0,
                                  0, 0, 1, None, None)
     assert rc == -1 and b"temperature" in lib.rlk_last_error()
