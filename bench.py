@@ -42,14 +42,14 @@ PEAK_HBM_GBS = 8000.0
 # the kernel sources whose digest is recorded with them; with other sources `traffic` is null.
 MEASURED_TRAFFIC = {
     "workload": "llama3-8b-head",
-    "kernel_source_sha16": "80eb8f1e8bf5f94f",
-    "measured_at_commit": "18862d0",
+    "kernel_source_sha16": "27f6927cb1dd4afa",
+    "measured_at_commit": "ed6874b",
     "counter_scale": {"FETCH_SIZE": 2.000, "WRITE_SIZE": 1.000},
     "bytes_per_launch": {
-        "linear_logp_fwd_kernel": 61219987021,
-        "linear_logp_dz_kernel": 1958503509,
-        "linear_logp_dh_kernel": 1851003309,
-        "linear_logp_dw_kernel": 2117548136,
+        "linear_logp_fwd_kernel": 57634103170,
+        "linear_logp_dz_kernel": 1958119534,
+        "linear_logp_dh_kernel": 1834437792,
+        "linear_logp_dw_kernel": 2108737019,
     },
 }
 
